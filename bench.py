@@ -1,0 +1,263 @@
+#!/usr/bin/env python3
+"""Benchmark of the CSR hot path on ONE MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config {1,2,3,4,5}]
+
+A step is one pass of the hot path over one batch of synthetic input resident in
+HBM: one SpMV (configs 1-3), one SpMM (config 4) or one CG iteration (config 5; a
+run is exactly `steps` iterations).  The default workload is config 2, the one the
+headline metric is quoted on.  Prints ONE JSON line.
+
+Protocol (benchmarks/spmv/main.cpp:52-62 of the reference): device-resident inputs,
+warm-up calls, then K calls; the K calls are timed as one region bracketed by device
+synchronisation, and the dominant kernel is timed per launch with HIP events
+attached to its dispatches in that same region.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def traffic_from_profiles(kernel_key):
+    """HBM bytes per launch measured with rocprofv3 --pmc (profiles/traffic.json), or None."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        return json.load(f).get(kernel_key, {}).get("hbm_bytes_per_launch")
+
+
+def cpu_baseline_spmv(A, x, budget_s=12.0):
+    """The OpenMP restatement of the reference loop nest, timed on this host's cores."""
+    from oracle.oracle import Oracle
+    omp = Oracle(omp=True)
+    y = np.zeros(A.nrows, dtype=A.val.dtype)
+    omp.spmv(A.pos, A.crd, A.val, x, y, parallel=True)  # warm-up, first touch
+    t0 = time.perf_counter()
+    omp.spmv(A.pos, A.crd, A.val, x, y, parallel=True)
+    one = time.perf_counter() - t0
+    reps = int(min(200, max(3, budget_s / max(one, 1e-6))))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        omp.spmv(A.pos, A.crd, A.val, x, y, parallel=True)
+    dt = (time.perf_counter() - t0) / reps
+    return {"value": A.spmv_bytes() / dt / 1e9, "unit": "GB/s", "cores": omp.max_threads(), "kind": "port",
+            "sample": "%d calls of the full workload (%d rows, %d non-zeros), OpenMP static row split, "
+                      "%.3f ms per call; Kokkos is not installed, so this is the C restatement of the "
+                      "reference loop nest" % (reps, A.nrows, A.nnz, dt * 1e3),
+            "gflops": 2.0 * A.nnz / dt / 1e9}
+
+
+def run_spmv(args, cfg):
+    import torch
+    from lapis_amd import generators as gen
+    from lapis_amd import hip
+    name, maker, dtype = {
+        1: ("config1: SpMV fp64, 2-D 5-point Laplacian 256x256", gen.config1, np.float64),
+        2: ("config2: SpMV fp64, n=4194304, Poisson(16) rows, uniform random sorted columns, int32 indices",
+            gen.config2, np.float64),
+        3: ("config3: SpMV fp32, n=2097152, power-law rows (exponent 2, min 1, cap 200000, mean 30)", gen.config3,
+            np.float32),
+    }[cfg]
+    t0 = time.perf_counter()
+    A, x = maker()
+    log("generated %s: %d rows, %d nnz in %.1f s" % (name, A.nrows, A.nnz, time.perf_counter() - t0))
+    dev = lambda a: torch.from_numpy(a).cuda()
+    pos, crd, val, dx = dev(A.pos), dev(A.crd), dev(A.val), dev(x)
+    y = torch.zeros(A.nrows, dtype=torch.float64 if dtype == np.float64 else torch.float32, device="cuda")
+    t0 = time.perf_counter()
+    plan = hip.CsrPlan(A.nrows, A.ncols, pos, crd, value_bytes=np.dtype(dtype).itemsize)
+    torch.cuda.synchronize()
+    plan_ms = (time.perf_counter() - t0) * 1e3
+    if args.kernel:
+        plan.set_kernel({"subwarp": 1, "rowblock": 2, "nnzsplit": 3}[args.kernel], args.width)
+    stats = plan.stats()
+    for _ in range(args.warmup):
+        hip.spmv(plan, A.nrows, A.ncols, pos, crd, val, dx, y)
+    torch.cuda.synchronize()
+    hip.kernel_timing_start(args.steps)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        hip.spmv(plan, A.nrows, A.ncols, pos, crd, val, dx, y)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    kt = hip.kernel_timing_stop()
+    bytes_step = A.spmv_bytes()
+    ms = elapsed / args.steps * 1e3
+    kernel_name = "spmv_%s_kernel<%s>" % (stats["kernel_name"], "double" if dtype == np.float64 else "float")
+    achieved = bytes_step / (kt["mean_ms"] * 1e-3) / 1e9
+    out = {
+        "metric": "CSR SpMV %s achieved HBM GB/s" % ("fp64" if dtype == np.float64 else "fp32"),
+        "value": bytes_step / (ms * 1e-3) / 1e9, "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f64" if dtype == np.float64 else "f32", "data": "synthetic",
+        "config": {"workload": name, "nrows": A.nrows, "nnz": A.nnz, "seed": {1: 1001, 2: 2002, 3: 3003}[cfg],
+                   "algorithmic_bytes_per_step": bytes_step, "kernel": stats["kernel_name"],
+                   "width": stats["width"], "chunk": stats["chunk"],
+                   "reference_vector_length": stats["reference_vector_length"], "plan_ms": plan_ms},
+        "pct_of_hbm_peak": 100.0 * bytes_step / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "gflops": 2.0 * A.nnz / (ms * 1e-3) / 1e9,
+        "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": achieved, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": traffic_from_profiles("%s_config%d" % (stats["kernel_name"], cfg)),
+                     "kernel_ms_mean": kt["mean_ms"], "kernel_ms_min": kt["min_ms"], "launches_timed": kt["count"]},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline_spmv(A, x)
+    return out
+
+
+def run_spmm(args):
+    import torch
+    from lapis_amd import generators as gen
+    from lapis_amd import hip
+    A, B = gen.config4()
+    k = B.shape[1]
+    dev = lambda a: torch.from_numpy(a).cuda()
+    pos, crd, val, dB = dev(A.pos), dev(A.crd), dev(A.val), dev(B)
+    C = torch.zeros(A.nrows, k, dtype=torch.float32, device="cuda")
+    for _ in range(args.warmup):
+        hip.spmm(A.nrows, A.ncols, pos, crd, val, dB, C)
+    torch.cuda.synchronize()
+    hip.kernel_timing_start(args.steps)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        hip.spmm(A.nrows, A.ncols, pos, crd, val, dB, C)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    kt = hip.kernel_timing_stop()
+    # A streamed once, B counted once, C written once (the read of C for the accumulate is not counted)
+    bytes_step = 8 * A.nnz + 4 * (A.nrows + 1) + 4 * A.ncols * k + 4 * A.nrows * k
+    ms = elapsed / args.steps * 1e3
+    achieved = bytes_step / (kt["mean_ms"] * 1e-3) / 1e9
+    out = {
+        "metric": "CSR x dense SpMM fp32 achieved HBM GB/s", "value": bytes_step / (ms * 1e-3) / 1e9, "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "config4: SpMM fp32, A 1048576^2 with 32 nnz/row, B 1048576x64 row-major",
+                   "nrows": A.nrows, "nnz": A.nnz, "k": k, "seed": 4004, "algorithmic_bytes_per_step": bytes_step},
+        "pct_of_hbm_peak": 100.0 * bytes_step / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "gflops": 2.0 * A.nnz * k / (ms * 1e-3) / 1e9,
+        "roofline": {"bound": "hbm", "kernel": "spmm_wave_row_kernel<float,16>", "achieved": achieved,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": traffic_from_profiles("spmm_config4"), "kernel_ms_mean": kt["mean_ms"],
+                     "launches_timed": kt["count"]},
+    }
+    if not args.no_cpu:
+        from oracle.oracle import Oracle
+        omp = Oracle(omp=True)
+        rows = A.nrows // 8  # bounded sample: the first eighth of the rows
+        sub_pos = A.pos[:rows + 1]
+        Cc = np.zeros((rows, k), np.float32)
+        t0 = time.perf_counter()
+        omp.spmm(sub_pos, A.crd, A.val, B, Cc, parallel=True)
+        dt = time.perf_counter() - t0
+        frac = rows / A.nrows
+        out["cpu_baseline"] = {"value": bytes_step * frac / dt / 1e9, "unit": "GB/s", "cores": omp.max_threads(),
+                               "kind": "port", "sample": "first %d of %d rows, one call, %.1f ms" % (rows, A.nrows, dt * 1e3)}
+    return out
+
+
+def run_cg(args):
+    import torch
+    from lapis_amd import generators as gen
+    from lapis_amd import hip
+    A, b = gen.config5()
+    n = A.nrows
+    dev = lambda a: torch.from_numpy(a).cuda()
+    pos, crd, val, db = dev(A.pos), dev(A.crd), dev(A.val), dev(b)
+    x = torch.empty(n, dtype=torch.float64, device="cuda")
+    work = torch.empty(4 * n, dtype=torch.float64, device="cuda")
+    plan = hip.CsrPlan(n, n, pos, crd)
+    hip.pcg(plan, n, pos, crd, val, db, None, 0.0, max(1, args.warmup), x, work=work)
+    torch.cuda.synchronize()
+    hip.kernel_timing_start(args.steps)
+    t0 = time.perf_counter()
+    iters, relres = hip.pcg(plan, n, pos, crd, val, db, None, 0.0, args.steps, x, work=work)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    kt = hip.kernel_timing_stop()
+    assert iters == args.steps
+    spmv_bytes = A.spmv_bytes()
+    bytes_step = spmv_bytes + 2 * 2 * 8 * n + 3 * 3 * 8 * n  # SpMV + 2 dots + 3 axpy
+    ms = elapsed / args.steps * 1e3
+    achieved = spmv_bytes / (kt["mean_ms"] * 1e-3) / 1e9
+    out = {
+        "metric": "CG fp64 achieved HBM GB/s per iteration", "value": bytes_step / (ms * 1e-3) / 1e9, "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic",
+        "config": {"workload": "config5: unpreconditioned CG fp64, 7-point Laplacian 192^3, %d iterations" % args.steps,
+                   "nrows": n, "nnz": A.nnz, "seed": 5005, "algorithmic_bytes_per_step": bytes_step,
+                   "final_relres": relres},
+        "pct_of_hbm_peak": 100.0 * bytes_step / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "gflops": (2.0 * A.nnz + 2 * 2 * n + 3 * 3 * n) / (ms * 1e-3) / 1e9,
+        "roofline": {"bound": "hbm", "kernel": "spmv_%s_kernel<double>" % plan.stats()["kernel_name"],
+                     "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": traffic_from_profiles("cg_spmv_config5"), "kernel_ms_mean": kt["mean_ms"],
+                     "launches_timed": kt["count"]},
+    }
+    if not args.no_cpu:
+        from oracle.oracle import Oracle
+        omp = Oracle(omp=True)
+        p, Ap = b.copy(), np.zeros(n)
+        reps = 3
+        t0 = time.perf_counter()
+        for _ in range(reps):  # one iteration's kernels: SpMV + 2 dots + 3 axpy
+            Ap[:] = 0
+            omp.spmv(A.pos, A.crd, A.val, p, Ap, parallel=True)
+            omp.dot(p, Ap, parallel=True)
+            omp.dot(Ap, Ap, parallel=True)
+            omp.axpby(1.0, p, 0.5, Ap, p, parallel=True)
+            omp.axpby(1.0, Ap, 0.5, p, Ap, parallel=True)
+            omp.axpby(1.0, p, 0.5, Ap, p, parallel=True)
+        dt = (time.perf_counter() - t0) / reps
+        out["cpu_baseline"] = {"value": bytes_step / dt / 1e9, "unit": "GB/s", "cores": omp.max_threads(), "kind": "port",
+                               "sample": "%d iterations' worth of SpMV + 2 dots + 3 axpy on the full workload" % reps}
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
+    ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5])
+    ap.add_argument("--kernel", choices=["subwarp", "rowblock", "nnzsplit"], default=None,
+                    help="force an SpMV kernel family instead of the plan's choice")
+    ap.add_argument("--width", type=int, default=0, help="lanes per row with --kernel subwarp (0 = the reference's rule)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+    if args.steps is None:
+        args.steps = {1: 1000, 2: 200, 3: 200, 4: 20, 5: 100}[args.config]
+    if args.warmup is None:
+        args.warmup = {1: 10, 2: 10, 3: 10, 4: 2, 5: 2}[args.config]
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU: the HIP library has no CPU path")
+    if args.config in (1, 2, 3):
+        out = run_spmv(args, args.config)
+    elif args.config == 4:
+        out = run_spmm(args)
+    else:
+        out = run_cg(args)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

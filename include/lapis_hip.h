@@ -1,0 +1,194 @@
+/*
+ * lapis_hip.h -- C ABI of the gfx950 (MI355X) kernel library behind
+ * LAPIS-generated sparse CSR modules.
+ *
+ * Every entry point takes plain DEVICE pointers and sizes, launches on the
+ * hipStream_t it is given (passed as void*, NULL = the null stream), returns a
+ * status code and never synchronises unless its comment says so.  Index
+ * buffers are int32 (posWidth = crdWidth = 32 of the reference's #sparse
+ * encoding, benchmarks/spmv/spmv.mlir:1).
+ *
+ * Each declaration names the piece of the reference whose emitted Kokkos code
+ * it replaces; paths are relative to the reference tree and
+ * "emitter" = mlir/lib/Target/KokkosCpp/TranslateToKokkosCpp.cpp.
+ */
+#ifndef LAPIS_HIP_H
+#define LAPIS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *lapis_hip_stream_t; /* a hipStream_t */
+
+enum lapis_hip_status {
+  LAPIS_HIP_OK = 0,
+  LAPIS_HIP_ERR_INVALID_ARGUMENT = 1, /* null pointer with non-zero size, negative size, bad enum */
+  LAPIS_HIP_ERR_RUNTIME = 2,          /* a HIP call or kernel launch failed */
+  LAPIS_HIP_ERR_NOT_INITIALIZED = 3,  /* lapis_hip_init() has not been called */
+  LAPIS_HIP_ERR_BAD_CSR = 4,          /* positions not monotone / coordinates out of range */
+  LAPIS_HIP_ERR_UNSUPPORTED_DEVICE = 5, /* the current device is not gfx950 */
+  LAPIS_HIP_ERR_PLAN_MISMATCH = 6     /* plan was built for other sizes or buffers */
+};
+
+/* ---- runtime ------------------------------------------------------------ */
+
+/* Replaces `if(!Kokkos::is_initialized()) Kokkos::initialize();` of the emitted
+ * lapis_initialize() (emitter :4284-4290).  Idempotent and reference counted;
+ * checks that the current device is gfx950. */
+int lapis_hip_init(void);
+/* Replaces `Kokkos::finalize()` of the emitted lapis_finalize() (emitter :4352-4376). */
+int lapis_hip_finalize(void);
+/* Message of the last non-OK status returned on the calling thread. */
+const char *lapis_hip_last_error(void);
+const char *lapis_hip_status_name(int status);
+/* Replaces Kokkos::DefaultExecutionSpace().fence() (emitter :2680-2682). */
+int lapis_hip_stream_synchronize(lapis_hip_stream_t stream);
+
+/* ---- kernel timing -------------------------------------------------------------- */
+
+/* Device-side duration of the dominant kernels (the SpMV main kernel of whichever
+ * family runs, and the SpMM kernel): between start and stop every such launch
+ * carries its own pair of HIP events, so the figure is the kernel's own run time
+ * on its stream, not a host clock.  The reference times whole fenced calls with
+ * Kokkos::Timer instead (benchmarks/spmv/main.cpp:52-62); these two calls exist
+ * for the roofline report only.  `capacity` = launches to keep (later ones are
+ * not timed).  stop synchronises the device and returns count / mean / min / max
+ * in milliseconds (any output may be NULL). */
+int lapis_hip_kernel_timing_start(int capacity);
+int lapis_hip_kernel_timing_stop(int *count, double *mean_ms, double *min_ms, double *max_ms);
+
+/* ---- CSR plan: the team/vector loop-mapping decision ---------------------- */
+
+/* Which kernel a plan launches for SpMV. */
+enum lapis_hip_spmv_kernel {
+  LAPIS_HIP_SPMV_AUTO = 0,
+  /* `width` lanes per row (1,2,4,...,64), rows packed into wave64; the shape the
+   * reference's TeamPolicy(league, team, vector) launch has (emitter :1976-2039). */
+  LAPIS_HIP_SPMV_SUBWARP = 1,
+  /* 64 consecutive rows per wavefront; their products are staged in LDS with
+   * 128-bit coalesced loads and summed one row per lane in ascending order. */
+  LAPIS_HIP_SPMV_ROWBLOCK = 2,
+  /* equal non-zero count per wavefront whatever the row lengths (row split);
+   * rows cut by a chunk boundary are completed by a small second kernel. */
+  LAPIS_HIP_SPMV_NNZSPLIT = 3
+};
+
+typedef struct lapis_hip_csr_stats {
+  int64_t nrows, ncols, nnz;
+  int64_t min_row_len, max_row_len, empty_rows;
+  double mean_row_len, var_row_len;
+  /* the reference's own decision for this matrix, for comparison:
+   * hint = ceil((pos[n]-pos[0])/n) (KokkosLoopMapping.cpp:279-323) and
+   * LAPIS::threadParallelVectorLength(hint) with vector_length_max = 64
+   * (LAPISSupport.hpp:428-435) */
+  int64_t reference_hint;
+  int32_t reference_vector_length;
+  /* what this plan launches */
+  int32_t kernel;      /* enum lapis_hip_spmv_kernel, never AUTO */
+  int32_t width;       /* lanes per row for SUBWARP, else 0 */
+  int32_t chunk;       /* non-zeros per wavefront for NNZSPLIT, else 0 */
+} lapis_hip_csr_stats;
+
+typedef struct lapis_hip_csr_plan lapis_hip_csr_plan;
+
+/* Replaces estimateParallelism + the nestingLevel==2 branch of the loop-mapping
+ * pass (KokkosLoopMapping.cpp:132-343, :888-921) and the per-launch
+ * team_size_recommended query (emitter :2013-2033): reads the row-length
+ * statistics of the matrix ONCE on the device, validates the structure
+ * (monotone positions, pos[0]==0, pos[n]==nnz, coordinates inside [0,ncols) when
+ * `crd` is non-NULL) and fixes the kernel.  `value_bytes` is 4 or 8.
+ * Synchronises `stream`.  The plan keeps `pos` by address: it stays valid for as
+ * long as that buffer holds the same positions. */
+int lapis_hip_csr_plan_create(lapis_hip_csr_plan **plan, int64_t nrows, int64_t ncols, int64_t nnz,
+                              const int32_t *pos, const int32_t *crd, int value_bytes,
+                              lapis_hip_stream_t stream);
+/* Overrides the automatic choice (tuning and tests).  `width` is used by SUBWARP
+ * (0 = the reference's rule); other kernels ignore it. */
+int lapis_hip_csr_plan_set_kernel(lapis_hip_csr_plan *plan, int kernel, int width);
+int lapis_hip_csr_plan_get_stats(const lapis_hip_csr_plan *plan, lapis_hip_csr_stats *stats);
+int lapis_hip_csr_plan_destroy(lapis_hip_csr_plan *plan);
+
+/* ---- SpMV ------------------------------------------------------------------ */
+
+/* y[i] = y[i] + sum_j val[j] * x[crd[j]],  j in [pos[i], pos[i+1]).
+ * Replaces the TeamPolicy/ThreadVectorRange lambda the emitter prints for
+ * tests/Dialect/Kokkos/loop_mapping_2.mlir.gold:12-37 (emitter :1966-2064 with
+ * :1692-1845, :2127-2157, :1671-1690, :2073-2125).
+ * `plan` may be NULL: the launch then follows the reference's rule, reading
+ * pos[n] and pos[0] back to the host on every call as the emitted code does
+ * (that read synchronises `stream`).  Calls sharing one plan must be ordered on
+ * one stream (the plan owns the row-split workspace).  x and y must not alias. */
+int lapis_hip_spmv_csr_f64_i32(lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols,
+                               const int32_t *pos, const int32_t *crd, const double *val,
+                               const double *x, double *y, lapis_hip_stream_t stream);
+int lapis_hip_spmv_csr_f32_i32(lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols,
+                               const int32_t *pos, const int32_t *crd, const float *val,
+                               const float *x, float *y, lapis_hip_stream_t stream);
+
+/* ---- SpMM ------------------------------------------------------------------ */
+
+/* C[i,:] = C[i,:] + sum_kk val[kk] * B[crd[kk],:]; B is ncols-by-k with leading
+ * dimension ldb, C is nrows-by-k with leading dimension ldc, both row-major.
+ * Replaces the nest the sparsifier emits for CSR x dense linalg.matmul
+ * (examples/spmm_dcsr_opdsl.py:73-110, examples/bspmm.py:22-50) under the
+ * race-free parallelization strategies (Pipelines/Passes.h:41-56). */
+int lapis_hip_spmm_csr_f32_i32(int64_t nrows, int64_t ncols, int64_t k, const int32_t *pos,
+                               const int32_t *crd, const float *val, const float *B, int64_t ldb,
+                               float *C, int64_t ldc, lapis_hip_stream_t stream);
+int lapis_hip_spmm_csr_f64_i32(int64_t nrows, int64_t ncols, int64_t k, const int32_t *pos,
+                               const int32_t *crd, const double *val, const double *B, int64_t ldb,
+                               double *C, int64_t ldc, lapis_hip_stream_t stream);
+
+/* ---- dense vector kernels of CG -------------------------------------------- */
+
+/* *result = init + sum_i x[i]*y[i]; `result` is a DEVICE scalar (no host sync,
+ * unlike the Kokkos::parallel_reduce into a host scalar it replaces: emitter
+ * :1696-1705, :1790-1844; loop shape tests/Dialect/Kokkos/linalg_to_loops_0.mlir.gold:7-18).
+ * Deterministic: fixed block partials summed in a fixed order. */
+int lapis_hip_dot_f64(int64_t n, const double *x, const double *y, double init, double *result,
+                      lapis_hip_stream_t stream);
+int lapis_hip_dot_f32(int64_t n, const float *x, const float *y, float init, float *result,
+                      lapis_hip_stream_t stream);
+/* dst[i] = a*x[i] + b*y[i] (examples/pcg_solve.py:30-38; RangePolicy parallel_for,
+ * emitter :1710-1715).  dst may alias x or y. */
+int lapis_hip_axpby_f64(int64_t n, double a, const double *x, double b, const double *y, double *dst,
+                        lapis_hip_stream_t stream);
+int lapis_hip_axpby_f32(int64_t n, float a, const float *x, float b, const float *y, float *dst,
+                        lapis_hip_stream_t stream);
+/* dst[i] = x[i]*y[i] (examples/pcg_solve.py:40-47). */
+int lapis_hip_mult_f64(int64_t n, const double *x, const double *y, double *dst, lapis_hip_stream_t stream);
+/* dst[i] = x[i]/y[i] (linalg.div of examples/hitting_times.py:120,146). */
+int lapis_hip_div_f64(int64_t n, const double *x, const double *y, double *dst, lapis_hip_stream_t stream);
+/* dst[i] = v (linalg.fill, examples/pcg_solve.py:15-17). */
+int lapis_hip_fill_f64(int64_t n, double v, double *dst, lapis_hip_stream_t stream);
+int lapis_hip_fill_f32(int64_t n, float v, float *dst, lapis_hip_stream_t stream);
+/* dst[i] = src[i] (linalg.copy, examples/pcg_solve.py:65-67). */
+int lapis_hip_copy_f64(int64_t n, const double *src, double *dst, lapis_hip_stream_t stream);
+/* val[j] *= alpha in place (scale_csr, examples/hitting_times.py:51-71). */
+int lapis_hip_scale_f64(int64_t n, double alpha, double *val, lapis_hip_stream_t stream);
+
+/* ---- CG -------------------------------------------------------------------- */
+
+/* The solver examples/pcg_solve.py:52-101 lowers to (host while-loop, emitter
+ * :1512-1593): x0 = 0, Jacobi preconditioner `dinv` (NULL = unpreconditioned:
+ * z = r, so the r.z and r.r products coincide and one iteration is
+ * SpMV + 2 dots + 3 axpy), stop when relres <= tol or the iteration counter,
+ * which starts at 1, equals maxiter.  All vectors are device buffers of length
+ * n; `work` is 4*n doubles of device scratch or NULL (allocated and freed
+ * inside).  Scalars stay on the device between kernels; the host looks at the
+ * convergence flag every few iterations only.  `iters` and `relres` are HOST
+ * outputs; the call synchronises `stream` before returning.
+ * `plan` may be NULL (one is built and destroyed inside). */
+int lapis_hip_pcg_f64_i32(lapis_hip_csr_plan *plan, int64_t n, const int32_t *pos, const int32_t *crd,
+                          const double *val, const double *b, const double *dinv, double tol,
+                          uint64_t maxiter, double *x, uint64_t *iters, double *relres, double *work,
+                          lapis_hip_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LAPIS_HIP_H */

@@ -1,0 +1,101 @@
+/*
+ * lapis_module.h -- the calling convention of a LAPIS-generated module, as
+ * exported by the prebuilt gfx950 module (liblapis_package_module.so).
+ *
+ * These are the symbols the reference's emitter writes into every generated
+ * module (mlir/lib/Target/KokkosCpp/TranslateToKokkosCpp.cpp, "emitter"):
+ *   lapis_initialize / lapis_finalize          emitter :4277-4378
+ *   py_<func>(results..., params...)           emitter :2541-2684
+ * Result slots come first; a memref result is StridedMemRefType<T,N>**, a
+ * scalar result T*; a memref parameter is StridedMemRefType<T,N>*, a sparse
+ * tensor's storage specifier is a struct of five int64 passed by reference
+ * ({dimSizes[2], memSizes[3]} = ((m, n), (m+1, nnz, nnz))), scalars by value.
+ * All buffers are HOST memory; a returned memref either aliases an input
+ * parameter (updated in place) or points at memory the module owns until
+ * lapis_finalize().  As in the reference there are no status codes: a memref
+ * that is not unit-stride, an invalid CSR structure or a failed HIP call prints
+ * a message and aborts.
+ */
+#ifndef LAPIS_MODULE_H
+#define LAPIS_MODULE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* StridedMemRefType<T,1> of mlir/lib/Target/KokkosCpp/LAPISSupport.hpp:7-14 */
+#define LAPIS_DECLARE_MEMREF_1D(NAME, T) \
+  typedef struct NAME {                  \
+    T *basePtr;                          \
+    T *data;                             \
+    int64_t offset;                      \
+    int64_t sizes[1];                    \
+    int64_t strides[1];                  \
+  } NAME
+
+LAPIS_DECLARE_MEMREF_1D(lapis_memref_1d_i32, int32_t);
+LAPIS_DECLARE_MEMREF_1D(lapis_memref_1d_f64, double);
+LAPIS_DECLARE_MEMREF_1D(lapis_memref_1d_f32, float);
+
+/* StridedMemRefType<T,2> */
+#define LAPIS_DECLARE_MEMREF_2D(NAME, T) \
+  typedef struct NAME {                  \
+    T *basePtr;                          \
+    T *data;                             \
+    int64_t offset;                      \
+    int64_t sizes[2];                    \
+    int64_t strides[2];                  \
+  } NAME
+
+LAPIS_DECLARE_MEMREF_2D(lapis_memref_2d_f32, float);
+LAPIS_DECLARE_MEMREF_2D(lapis_memref_2d_f64, double);
+
+/* storage specifier of a decomposed 2-D CSR tensor (benchmarks/spmv/main.cpp:48-51) */
+typedef struct lapis_csr_specifier {
+  int64_t dimSizes[2];
+  int64_t memSizes[3];
+} lapis_csr_specifier;
+
+void lapis_initialize(void);
+void lapis_finalize(void);
+
+/* func @spmv(A, x, y) -> y of examples/spmv_noalloc.py:9-14 and
+ * benchmarks/spmv/spmv.mlir:3-6: y += A*x, y updated in place and returned. */
+void py_spmv(lapis_memref_1d_f64 **ret0, lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd,
+             lapis_memref_1d_f64 *val, const lapis_csr_specifier *spec, lapis_memref_1d_f64 *x,
+             lapis_memref_1d_f64 *y);
+
+/* the fp32 instance of the same function (config 3 of the benchmark set) */
+void py_spmv_f32(lapis_memref_1d_f32 **ret0, lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd,
+                 lapis_memref_1d_f32 *val, const lapis_csr_specifier *spec, lapis_memref_1d_f32 *x,
+                 lapis_memref_1d_f32 *y);
+
+/* torch.mv export of examples/spmv.py:13-18,47 (entry `main` is renamed
+ * lapis_main, emitter :2351-2355): y = A*x with y allocated by the module. */
+void py_lapis_main(lapis_memref_1d_f64 **ret0, lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd,
+                   lapis_memref_1d_f64 *val, const lapis_csr_specifier *spec, lapis_memref_1d_f64 *x);
+
+/* func @pcg(A, b, dinv, tol, maxiter) -> (x, iters, relres) of examples/pcg_solve.py:52. */
+void py_pcg(lapis_memref_1d_f64 **ret0, size_t *ret1, double *ret2, lapis_memref_1d_i32 *pos,
+            lapis_memref_1d_i32 *crd, lapis_memref_1d_f64 *val, const lapis_csr_specifier *spec,
+            lapis_memref_1d_f64 *b, lapis_memref_1d_f64 *dinv, double tol, size_t maxiter);
+
+/* CSR x dense matmul, C += A*B with C updated in place and returned (the
+ * decomposed-CSR form of spMxM, examples/spmm_dcsr_opdsl.py:73-110). */
+void py_spmm(lapis_memref_2d_f32 **ret0, lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd,
+             lapis_memref_1d_f32 *val, const lapis_csr_specifier *spec, lapis_memref_2d_f32 *B,
+             lapis_memref_2d_f32 *C);
+void py_spmm_f64(lapis_memref_2d_f64 **ret0, lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd,
+                 lapis_memref_1d_f64 *val, const lapis_csr_specifier *spec, lapis_memref_2d_f64 *B,
+                 lapis_memref_2d_f64 *C);
+
+/* func @plus_norm(x, y) -> (x+y, ||x+y||) of examples/multiple_results.py:8-19. */
+void py_plus_norm(lapis_memref_1d_f64 **ret0, double *ret1, lapis_memref_1d_f64 *x, lapis_memref_1d_f64 *y);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LAPIS_MODULE_H */

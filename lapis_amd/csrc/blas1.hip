@@ -1,0 +1,244 @@
+// Dense vector kernels of the CG path: dot, axpby, mult, div, fill, copy, scale.
+// They replace the RangePolicy parallel_for / parallel_reduce launches the
+// reference emits for the linalg.generic / linalg.dot ops of
+// examples/pcg_solve.py:22-47.
+#include <mutex>
+
+#include "blas1.hpp"
+#include "common.hpp"
+
+namespace lapis {
+
+// ---- elementwise ----------------------------------------------------------------
+// One pass; each thread takes VW consecutive elements with one 128-bit access when
+// every buffer is 16-byte aligned, the last n % VW elements go to the tail threads.
+template <typename T>
+struct VecOf;
+template <>
+struct VecOf<double> {
+  typedef v2d type;
+  static constexpr int width = 2;
+};
+template <>
+struct VecOf<float> {
+  typedef v4f type;
+  static constexpr int width = 4;
+};
+
+template <typename T, typename F, int NIN>
+__global__ __launch_bounds__(256) void elementwise_kernel(long long n, long long nvec, const T *a, const T *b,
+                                                          T *dst, F f) {
+  typedef typename VecOf<T>::type V;
+  constexpr int VW = VecOf<T>::width;
+  const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (t < nvec) {
+    V va = {}, vb = {}, vo;
+    if (NIN >= 1) va = reinterpret_cast<const V *>(a)[t];
+    if (NIN >= 2) vb = reinterpret_cast<const V *>(b)[t];
+#pragma unroll
+    for (int e = 0; e < VW; ++e) vo[e] = f(va[e], vb[e]);
+    reinterpret_cast<V *>(dst)[t] = vo;
+  } else {
+    const long long i = nvec * VW + (t - nvec);
+    if (i < n) {
+      const T xa = NIN >= 1 ? a[i] : T(0);
+      const T xb = NIN >= 2 ? b[i] : T(0);
+      dst[i] = f(xa, xb);
+    }
+  }
+}
+
+template <typename T, int NIN, typename F>
+int launch_elementwise(const char *what, int64_t n, const T *a, const T *b, T *dst, F f, hipStream_t st) {
+  LAPIS_CHECK_INIT();
+  LAPIS_REQUIRE(n >= 0, "%s: negative length", what);
+  if (n == 0) return LAPIS_HIP_OK;
+  LAPIS_REQUIRE(dst && (NIN < 1 || a) && (NIN < 2 || b), "%s: null buffer with n=%lld", what, (long long)n);
+  constexpr int VW = VecOf<T>::width;
+  const bool vec = aligned16(dst) && (NIN < 1 || aligned16(a)) && (NIN < 2 || aligned16(b));
+  const long long nvec = vec ? n / VW : 0;
+  const long long threads = nvec + (n - nvec * VW);
+  const long long blocks = ceil_div(threads, 256);
+  LAPIS_REQUIRE(blocks <= 0x7fffffffLL, "%s: n=%lld exceeds the grid limit", what, (long long)n);
+  hipLaunchKernelGGL((elementwise_kernel<T, F, NIN>), dim3((unsigned)blocks), dim3(256), 0, st, (long long)n,
+                     nvec, a, b, dst, f);
+  LAPIS_LAUNCH_CHECK();
+  return LAPIS_HIP_OK;
+}
+
+template <typename T>
+struct AxpbyOp {
+  T a, b;
+  // x*a and y*b are rounded separately, then added (examples/pcg_solve.py:33-35)
+  __device__ T operator()(T x, T y) const {
+    const T t0 = x * a;
+    const T t1 = y * b;
+    return t0 + t1;
+  }
+};
+template <typename T>
+struct MultOp {
+  __device__ T operator()(T x, T y) const { return x * y; }
+};
+template <typename T>
+struct DivOp {
+  __device__ T operator()(T x, T y) const { return x / y; }
+};
+template <typename T>
+struct FillOp {
+  T v;
+  __device__ T operator()(T, T) const { return v; }
+};
+template <typename T>
+struct CopyOp {
+  __device__ T operator()(T x, T) const { return x; }
+};
+template <typename T>
+struct ScaleOp {
+  T a;
+  __device__ T operator()(T x, T) const { return x * a; }
+};
+
+// ---- dot --------------------------------------------------------------------------
+// Stage 1: each block sums a grid-strided slice (per-thread partial, DPP wave sum,
+// LDS across the waves in wave order) into partials[block].  The block that takes
+// the last ticket sums partials[] in index order and writes init + total, so the
+// result is the same from run to run.
+template <typename T>
+__device__ __forceinline__ T block_sum_256(T v, T *lds4) {
+  v = group_sum<64>(v);
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) lds4[wave] = v;
+  __syncthreads();
+  const T total = ((lds4[0] + lds4[1]) + lds4[2]) + lds4[3];
+  __syncthreads();
+  return total;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void dot_kernel(long long n, const T *__restrict__ x, const T *__restrict__ y,
+                                                  T init, T *partials, unsigned *ticket,
+                                                  T *__restrict__ result) {
+  __shared__ T lds4[4];
+  __shared__ bool is_last;
+  T acc = T(0);
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
+    acc = acc + x[i] * y[i];
+  const T total = block_sum_256(acc, lds4);
+  if (threadIdx.x == 0) {
+    partials[blockIdx.x] = total;
+    __threadfence();
+    const unsigned t = atomicAdd(ticket, 1u);
+    is_last = (t == gridDim.x - 1);
+  }
+  __syncthreads();
+  if (!is_last) return;
+  __threadfence();
+  T s = T(0);
+  for (unsigned i = threadIdx.x; i < gridDim.x; i += 256) s = s + partials[i];
+  const T all = block_sum_256(s, lds4);
+  if (threadIdx.x == 0) {
+    *result = all + init;
+    *ticket = 0u;
+  }
+}
+
+int dot_grid(int64_t n) {
+  const int64_t want = ceil_div(n, 256 * 8);
+  const int64_t cap = std::max(1, device_cu_count()) * 8;
+  return (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(want, cap), kDotMaxBlocks));
+}
+
+template <typename T>
+int launch_dot(int64_t n, const T *x, const T *y, T init, T *result, T *partials, unsigned *ticket,
+               hipStream_t st) {
+  hipLaunchKernelGGL((dot_kernel<T>), dim3(dot_grid(n)), dim3(256), 0, st, (long long)n, x, y, init, partials,
+                     ticket, result);
+  LAPIS_LAUNCH_CHECK();
+  return LAPIS_HIP_OK;
+}
+template int launch_dot<double>(int64_t, const double *, const double *, double, double *, double *, unsigned *,
+                                hipStream_t);
+template int launch_dot<float>(int64_t, const float *, const float *, float, float *, float *, unsigned *,
+                               hipStream_t);
+
+// Scratch for the stand-alone dot entry points: a ring of slots, one per call, so
+// that dots queued on different streams do not share partials unless more than
+// kSlots of them are in flight at once.
+namespace {
+constexpr int kSlots = 64;
+std::mutex g_scratch_mutex;
+char *g_scratch = nullptr;  // kSlots * (kDotMaxBlocks * 8 + 256) bytes
+unsigned g_next_slot = 0;
+constexpr size_t kSlotBytes = (size_t)kDotMaxBlocks * 8 + 256;
+
+int take_slot(void **partials, unsigned **ticket) {
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch) {
+    LAPIS_HIP_TRY(hipMalloc(&g_scratch, kSlots * kSlotBytes));
+    LAPIS_HIP_TRY(hipMemset(g_scratch, 0, kSlots * kSlotBytes));
+  }
+  char *slot = g_scratch + (size_t)(g_next_slot++ % kSlots) * kSlotBytes;
+  *partials = slot;
+  *ticket = reinterpret_cast<unsigned *>(slot + (size_t)kDotMaxBlocks * 8);
+  return LAPIS_HIP_OK;
+}
+
+template <typename T>
+int dot_entry(const char *what, int64_t n, const T *x, const T *y, T init, T *result, lapis_hip_stream_t stream) {
+  LAPIS_CHECK_INIT();
+  LAPIS_REQUIRE(n >= 0, "%s: negative length", what);
+  LAPIS_REQUIRE(result, "%s: null result", what);
+  LAPIS_REQUIRE(n == 0 || (x && y), "%s: null vector with n=%lld", what, (long long)n);
+  void *partials = nullptr;
+  unsigned *ticket = nullptr;
+  const int rc = take_slot(&partials, &ticket);
+  if (rc != LAPIS_HIP_OK) return rc;
+  return launch_dot<T>(n, x, y, init, result, static_cast<T *>(partials), ticket, as_stream(stream));
+}
+}  // namespace
+
+}  // namespace lapis
+
+using namespace lapis;
+
+extern "C" int lapis_hip_dot_f64(int64_t n, const double *x, const double *y, double init, double *result,
+                                 lapis_hip_stream_t stream) {
+  return dot_entry<double>("dot_f64", n, x, y, init, result, stream);
+}
+extern "C" int lapis_hip_dot_f32(int64_t n, const float *x, const float *y, float init, float *result,
+                                 lapis_hip_stream_t stream) {
+  return dot_entry<float>("dot_f32", n, x, y, init, result, stream);
+}
+extern "C" int lapis_hip_axpby_f64(int64_t n, double a, const double *x, double b, const double *y, double *dst,
+                                   lapis_hip_stream_t stream) {
+  return launch_elementwise<double, 2>("axpby_f64", n, x, y, dst, AxpbyOp<double>{a, b}, as_stream(stream));
+}
+extern "C" int lapis_hip_axpby_f32(int64_t n, float a, const float *x, float b, const float *y, float *dst,
+                                   lapis_hip_stream_t stream) {
+  return launch_elementwise<float, 2>("axpby_f32", n, x, y, dst, AxpbyOp<float>{a, b}, as_stream(stream));
+}
+extern "C" int lapis_hip_mult_f64(int64_t n, const double *x, const double *y, double *dst,
+                                  lapis_hip_stream_t stream) {
+  return launch_elementwise<double, 2>("mult_f64", n, x, y, dst, MultOp<double>{}, as_stream(stream));
+}
+extern "C" int lapis_hip_div_f64(int64_t n, const double *x, const double *y, double *dst,
+                                 lapis_hip_stream_t stream) {
+  return launch_elementwise<double, 2>("div_f64", n, x, y, dst, DivOp<double>{}, as_stream(stream));
+}
+extern "C" int lapis_hip_fill_f64(int64_t n, double v, double *dst, lapis_hip_stream_t stream) {
+  return launch_elementwise<double, 0>("fill_f64", n, (const double *)nullptr, (const double *)nullptr, dst,
+                                       FillOp<double>{v}, as_stream(stream));
+}
+extern "C" int lapis_hip_fill_f32(int64_t n, float v, float *dst, lapis_hip_stream_t stream) {
+  return launch_elementwise<float, 0>("fill_f32", n, (const float *)nullptr, (const float *)nullptr, dst,
+                                      FillOp<float>{v}, as_stream(stream));
+}
+extern "C" int lapis_hip_copy_f64(int64_t n, const double *src, double *dst, lapis_hip_stream_t stream) {
+  return launch_elementwise<double, 1>("copy_f64", n, src, (const double *)nullptr, dst, CopyOp<double>{},
+                                       as_stream(stream));
+}
+extern "C" int lapis_hip_scale_f64(int64_t n, double alpha, double *val, lapis_hip_stream_t stream) {
+  return launch_elementwise<double, 1>("scale_f64", n, val, (const double *)nullptr, val, ScaleOp<double>{alpha},
+                                       as_stream(stream));
+}

@@ -1,0 +1,20 @@
+// Internal interface of the dot kernel, shared with the CG driver.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace lapis {
+
+constexpr int kDotMaxBlocks = 2048;  // upper bound of dot_grid(); sizes the partials scratch
+
+// Number of blocks (= partial sums) a dot over n elements uses.
+int dot_grid(int64_t n);
+
+// *result = init + sum x[i]*y[i].  `partials` holds kDotMaxBlocks elements of T,
+// `*ticket` must be 0 on entry and is 0 again on exit.
+template <typename T>
+int launch_dot(int64_t n, const T *x, const T *y, T init, T *result, T *partials, unsigned *ticket,
+               hipStream_t st);
+
+}  // namespace lapis

@@ -1,0 +1,122 @@
+// Shared host/device helpers of the gfx950 kernel library.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "lapis_hip.h"
+
+namespace lapis {
+
+constexpr int kWave = 64;  // CDNA wavefront width
+
+// ---- host: status and error text ---------------------------------------------
+int set_error(int status, const char *fmt, ...);
+bool is_initialized();
+
+#define LAPIS_CHECK_INIT()                                                          \
+  do {                                                                              \
+    if (!::lapis::is_initialized())                                                 \
+      return ::lapis::set_error(LAPIS_HIP_ERR_NOT_INITIALIZED,                      \
+                                "%s: lapis_hip_init() has not been called", __func__); \
+  } while (0)
+
+#define LAPIS_HIP_TRY(expr)                                                         \
+  do {                                                                              \
+    hipError_t e_ = (expr);                                                         \
+    if (e_ != hipSuccess)                                                           \
+      return ::lapis::set_error(LAPIS_HIP_ERR_RUNTIME, "%s: %s failed: %s", __func__, #expr, \
+                                hipGetErrorString(e_));                             \
+  } while (0)
+
+#define LAPIS_LAUNCH_CHECK() LAPIS_HIP_TRY(hipGetLastError())
+
+#define LAPIS_REQUIRE(cond, ...)                                                    \
+  do {                                                                              \
+    if (!(cond)) return ::lapis::set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT, __VA_ARGS__); \
+  } while (0)
+
+inline hipStream_t as_stream(lapis_hip_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+int device_cu_count();
+
+// Event pair for the next launch of a dominant kernel while kernel timing is on
+// (see lapis_hip_kernel_timing_start); false when timing is off or the ring is full.
+bool timing_next_events(hipEvent_t *start, hipEvent_t *stop);
+
+// Launches `kernel`, attaching a start/stop event pair to the dispatch when kernel
+// timing is on.
+template <typename... KArgs, typename... Args>
+inline void launch_timed(void (*kernel)(KArgs...), dim3 grid, dim3 block, hipStream_t st, Args... args) {
+  hipEvent_t e0, e1;
+  if (timing_next_events(&e0, &e1))
+    hipExtLaunchKernelGGL(kernel, grid, block, 0, st, e0, e1, 0, args...);
+  else
+    hipLaunchKernelGGL(kernel, grid, block, 0, st, args...);
+}
+
+// ---- device: vector types, streaming loads ------------------------------------
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef double v2d __attribute__((ext_vector_type(2)));
+
+// Streamed-once data (crd, val, pos) is loaded non-temporally so that it does not
+// displace the gathered vector x from L2.
+template <typename V>
+__device__ __forceinline__ V load_stream(const V *p) {
+  return __builtin_nontemporal_load(p);
+}
+template <typename V>
+__device__ __forceinline__ void store_stream(V *p, V v) {
+  __builtin_nontemporal_store(v, p);
+}
+
+// ---- device: DPP wavefront reductions -------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ int dpp_mov(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, false);
+}
+template <int CTRL>
+__device__ __forceinline__ float dpp_get(float v) {
+  return __builtin_bit_cast(float, dpp_mov<CTRL>(__builtin_bit_cast(int, v)));
+}
+template <int CTRL>
+__device__ __forceinline__ double dpp_get(double v) {
+  v2i w = __builtin_bit_cast(v2i, v);
+  w.x = dpp_mov<CTRL>(w.x);
+  w.y = dpp_mov<CTRL>(w.y);
+  return __builtin_bit_cast(double, w);
+}
+
+// Sum over aligned groups of W consecutive lanes; every lane of a group ends with
+// the group's total.  Steps inside a 16-lane DPP row use quad_perm / row mirrors
+// (no LDS traffic); the 32- and 64-lane steps cross rows with a bpermute.
+template <int W, typename T>
+__device__ __forceinline__ T group_sum(T v) {
+  static_assert(W >= 1 && W <= 64 && (W & (W - 1)) == 0, "W must be a power of two <= 64");
+  if (W >= 2) v = v + dpp_get<0xB1>(v);   // quad_perm [1,0,3,2]
+  if (W >= 4) v = v + dpp_get<0x4E>(v);   // quad_perm [2,3,0,1]
+  if (W >= 8) v = v + dpp_get<0x141>(v);  // row_half_mirror
+  if (W >= 16) v = v + dpp_get<0x140>(v); // row_mirror
+  if (W >= 32) v = v + __shfl_xor(v, 16, 64);
+  if (W >= 64) v = v + __shfl_xor(v, 32, 64);
+  return v;
+}
+
+// Orders LDS traffic between the lanes of ONE wavefront (no s_barrier): LDS
+// operations of a wave execute in issue order, the fences stop the compiler from
+// moving accesses across this point.
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+}  // namespace lapis

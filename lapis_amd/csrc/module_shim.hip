@@ -1,0 +1,303 @@
+// The generated-module calling convention (lapis_initialize / lapis_finalize /
+// py_<func> over StridedMemRefType descriptors of HOST buffers) on top of the
+// gfx950 kernel library.  This file plays the role of the C++ a LAPIS module is
+// emitted as: the py_ wrappers (TranslateToKokkosCpp.cpp:2541-2684), the
+// host<->device mirroring of LAPIS::DualView (LAPISSupport.hpp:136-426) and the
+// keep-alive list for results handed to Python (LAPISSupport.hpp:101-120).
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <memory>
+#include <mutex>
+#include <vector>
+
+#include "lapis_hip.h"
+#include "lapis_module.h"
+
+namespace {
+
+[[noreturn]] void module_abort(const char *msg) {
+  // the counterpart of Kokkos::abort (LAPISSupport.hpp:76,86): no status channel exists
+  fprintf(stderr, "lapis module: %s\n", msg);
+  fflush(stderr);
+  abort();
+}
+
+void check(int status, const char *what) {
+  if (status != LAPIS_HIP_OK) {
+    char buf[768];
+    snprintf(buf, sizeof(buf), "%s failed: %s (%s)", what, lapis_hip_status_name(status), lapis_hip_last_error());
+    module_abort(buf);
+  }
+}
+
+void check_hip(hipError_t e, const char *what) {
+  if (e != hipSuccess) {
+    char buf[512];
+    snprintf(buf, sizeof(buf), "%s failed: %s", what, hipGetErrorString(e));
+    module_abort(buf);
+  }
+}
+
+// Results returned to Python stay allocated until lapis_finalize().
+std::mutex g_mutex;
+std::vector<void *> g_alives;
+int g_initialized = 0;
+
+void *keep_alive_alloc(size_t bytes) {
+  void *p = malloc(bytes ? bytes : 1);
+  if (!p) module_abort("out of host memory for a result");
+  std::lock_guard<std::mutex> lock(g_mutex);
+  g_alives.push_back(p);
+  return p;
+}
+
+// stridedMemrefToView<LayoutRight> (LAPISSupport.hpp:36-91): unit innermost stride,
+// each outer stride the product of the inner extents, else abort.
+template <typename M>
+auto *host_data(const M *m, int rank, const char *name) {
+  int64_t expected = 1;
+  for (int i = rank - 1; i >= 0; --i) {
+    if (m->strides[i] != expected) {
+      char buf[256];
+      snprintf(buf, sizeof(buf),
+               "Cannot shallow-copy StridedMemRefType that is not contiguous and LayoutRight (%s)", name);
+      module_abort(buf);
+    }
+    expected *= m->sizes[i];
+  }
+  return m->data + m->offset;
+}
+
+// The device half of a DualView built from a host view: allocated and filled from
+// the host buffer at construction ("modified_host" then syncDevice), copied back on
+// request (syncHost), freed at scope exit.
+template <typename T>
+struct DeviceMirror {
+  T *dev = nullptr;
+  T *host = nullptr;
+  size_t count = 0;
+  DeviceMirror() = default;
+  DeviceMirror(T *h, size_t n, bool upload = true) : host(h), count(n) {
+    if (n == 0) return;
+    check_hip(hipMalloc(&dev, n * sizeof(T)), "hipMalloc");
+    if (upload) check_hip(hipMemcpy(dev, h, n * sizeof(T), hipMemcpyHostToDevice), "host-to-device copy");
+  }
+  DeviceMirror(const DeviceMirror &) = delete;
+  DeviceMirror &operator=(const DeviceMirror &) = delete;
+  ~DeviceMirror() {
+    if (dev) (void)hipFree(dev);
+  }
+  void sync_host() {
+    if (count) check_hip(hipMemcpy(host, dev, count * sizeof(T), hipMemcpyDeviceToHost), "device-to-host copy");
+  }
+};
+
+template <typename M, typename T>
+void set_result_1d(M **ret, T *data, int64_t n) {
+  (*ret)->basePtr = data;
+  (*ret)->data = data;
+  (*ret)->offset = 0;
+  (*ret)->sizes[0] = n;
+  (*ret)->strides[0] = 1;
+}
+
+struct CsrArgs {
+  int64_t nrows, ncols, nnz;
+};
+
+CsrArgs csr_args(const lapis_memref_1d_i32 *pos, const lapis_memref_1d_i32 *crd, int64_t val_size,
+                 const lapis_csr_specifier *spec) {
+  CsrArgs a;
+  a.nrows = spec->dimSizes[0];
+  a.ncols = spec->dimSizes[1];
+  if (a.nrows < 0 || a.ncols < 0) module_abort("negative dimension in the storage specifier");
+  if (pos->sizes[0] < a.nrows + 1) module_abort("positions buffer shorter than rows+1");
+  const int32_t *p = pos->data + pos->offset;
+  a.nnz = p[a.nrows];
+  if (a.nnz < 0 || crd->sizes[0] < a.nnz || val_size < a.nnz)
+    module_abort("coordinates/values buffer shorter than pos[rows]");
+  return a;
+}
+
+template <typename T, typename MV>
+void spmv_entry(MV **ret0, lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd, MV *val,
+                const lapis_csr_specifier *spec, MV *x, MV *y, bool allocate_y) {
+  int32_t *hpos = host_data(pos, 1, "positions");
+  int32_t *hcrd = host_data(crd, 1, "coordinates");
+  T *hval = host_data(val, 1, "values");
+  T *hx = host_data(x, 1, "x");
+  const CsrArgs a = csr_args(pos, crd, val->sizes[0], spec);
+  if (x->sizes[0] < a.ncols) module_abort("x is shorter than the number of columns");
+  T *hy = nullptr;
+  if (allocate_y) {
+    // the torch.mv export allocates and zero-fills its result inside the function
+    hy = static_cast<T *>(keep_alive_alloc(sizeof(T) * (size_t)a.nrows));
+    memset(hy, 0, sizeof(T) * (size_t)a.nrows);
+  } else {
+    hy = host_data(y, 1, "y");
+    if (y->sizes[0] < a.nrows) module_abort("y is shorter than the number of rows");
+  }
+  {
+    DeviceMirror<int32_t> dpos(hpos, (size_t)a.nrows + 1), dcrd(hcrd, (size_t)a.nnz);
+    DeviceMirror<T> dval(hval, (size_t)a.nnz), dx(hx, (size_t)a.ncols), dy(hy, (size_t)a.nrows);
+    lapis_hip_csr_plan *plan = nullptr;
+    check(lapis_hip_csr_plan_create(&plan, a.nrows, a.ncols, a.nnz, dpos.dev, dcrd.dev, (int)sizeof(T), nullptr),
+          "lapis_hip_csr_plan_create");
+    int rc;
+    if (sizeof(T) == 8)
+      rc = lapis_hip_spmv_csr_f64_i32(plan, a.nrows, a.ncols, dpos.dev, dcrd.dev, (const double *)dval.dev,
+                                      (const double *)dx.dev, (double *)dy.dev, nullptr);
+    else
+      rc = lapis_hip_spmv_csr_f32_i32(plan, a.nrows, a.ncols, dpos.dev, dcrd.dev, (const float *)dval.dev,
+                                      (const float *)dx.dev, (float *)dy.dev, nullptr);
+    check(rc, "lapis_hip_spmv_csr");
+    check(lapis_hip_stream_synchronize(nullptr), "stream synchronize");
+    lapis_hip_csr_plan_destroy(plan);
+    dy.sync_host();  // results.syncHost(): the caller's y (or the module's) now holds the result
+  }
+  set_result_1d(ret0, hy, a.nrows);
+}
+
+template <typename T, typename MV, typename MM>
+void spmm_entry(MM **ret0, lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd, MV *val,
+                const lapis_csr_specifier *spec, MM *B, MM *C) {
+  int32_t *hpos = host_data(pos, 1, "positions");
+  int32_t *hcrd = host_data(crd, 1, "coordinates");
+  T *hval = host_data(val, 1, "values");
+  T *hB = host_data(B, 2, "B");
+  T *hC = host_data(C, 2, "C");
+  const CsrArgs a = csr_args(pos, crd, val->sizes[0], spec);
+  const int64_t k = C->sizes[1];
+  if (B->sizes[0] < a.ncols || B->sizes[1] != k || C->sizes[0] < a.nrows)
+    module_abort("SpMM operand shapes do not agree");
+  {
+    DeviceMirror<int32_t> dpos(hpos, (size_t)a.nrows + 1), dcrd(hcrd, (size_t)a.nnz);
+    DeviceMirror<T> dval(hval, (size_t)a.nnz), dB(hB, (size_t)(a.ncols * k)), dC(hC, (size_t)(a.nrows * k));
+    // the plan is built only for its structure check: a bad coordinate must not reach the kernel
+    lapis_hip_csr_plan *plan = nullptr;
+    check(lapis_hip_csr_plan_create(&plan, a.nrows, a.ncols, a.nnz, dpos.dev, dcrd.dev, (int)sizeof(T), nullptr),
+          "lapis_hip_csr_plan_create");
+    lapis_hip_csr_plan_destroy(plan);
+    int rc;
+    if (sizeof(T) == 8)
+      rc = lapis_hip_spmm_csr_f64_i32(a.nrows, a.ncols, k, dpos.dev, dcrd.dev, (const double *)dval.dev,
+                                      (const double *)dB.dev, k, (double *)dC.dev, k, nullptr);
+    else
+      rc = lapis_hip_spmm_csr_f32_i32(a.nrows, a.ncols, k, dpos.dev, dcrd.dev, (const float *)dval.dev,
+                                      (const float *)dB.dev, k, (float *)dC.dev, k, nullptr);
+    check(rc, "lapis_hip_spmm_csr");
+    check(lapis_hip_stream_synchronize(nullptr), "stream synchronize");
+    dC.sync_host();
+  }
+  (*ret0)->basePtr = hC;
+  (*ret0)->data = hC;
+  (*ret0)->offset = 0;
+  (*ret0)->sizes[0] = C->sizes[0];
+  (*ret0)->sizes[1] = k;
+  (*ret0)->strides[0] = k;
+  (*ret0)->strides[1] = 1;
+}
+
+}  // namespace
+
+extern "C" void lapis_initialize(void) {
+  std::lock_guard<std::mutex> lock(g_mutex);
+  if (g_initialized) return;  // `if (!Kokkos::is_initialized())`: repeated calls do nothing
+  check(lapis_hip_init(), "lapis_hip_init");
+  g_initialized = 1;
+}
+
+extern "C" void lapis_finalize(void) {
+  std::lock_guard<std::mutex> lock(g_mutex);
+  for (void *p : g_alives) free(p);  // LAPIS::alives.clear()
+  g_alives.clear();
+  if (g_initialized) {
+    lapis_hip_finalize();
+    g_initialized = 0;
+  }
+}
+
+extern "C" void py_spmv(lapis_memref_1d_f64 **ret0, lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd,
+                        lapis_memref_1d_f64 *val, const lapis_csr_specifier *spec, lapis_memref_1d_f64 *x,
+                        lapis_memref_1d_f64 *y) {
+  spmv_entry<double>(ret0, pos, crd, val, spec, x, y, false);
+}
+
+extern "C" void py_spmv_f32(lapis_memref_1d_f32 **ret0, lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd,
+                            lapis_memref_1d_f32 *val, const lapis_csr_specifier *spec, lapis_memref_1d_f32 *x,
+                            lapis_memref_1d_f32 *y) {
+  spmv_entry<float>(ret0, pos, crd, val, spec, x, y, false);
+}
+
+extern "C" void py_lapis_main(lapis_memref_1d_f64 **ret0, lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd,
+                              lapis_memref_1d_f64 *val, const lapis_csr_specifier *spec, lapis_memref_1d_f64 *x) {
+  spmv_entry<double>(ret0, pos, crd, val, spec, x, (lapis_memref_1d_f64 *)nullptr, true);
+}
+
+extern "C" void py_pcg(lapis_memref_1d_f64 **ret0, size_t *ret1, double *ret2, lapis_memref_1d_i32 *pos,
+                       lapis_memref_1d_i32 *crd, lapis_memref_1d_f64 *val, const lapis_csr_specifier *spec,
+                       lapis_memref_1d_f64 *b, lapis_memref_1d_f64 *dinv, double tol, size_t maxiter) {
+  int32_t *hpos = host_data(pos, 1, "positions");
+  int32_t *hcrd = host_data(crd, 1, "coordinates");
+  double *hval = host_data(val, 1, "values");
+  double *hb = host_data(b, 1, "b");
+  double *hdinv = host_data(dinv, 1, "dinv");
+  const CsrArgs a = csr_args(pos, crd, val->sizes[0], spec);
+  const int64_t n = b->sizes[0];  // %n = tensor.dim %b (examples/pcg_solve.py:55)
+  if (a.nrows != n || a.ncols != n || dinv->sizes[0] < n) module_abort("pcg: A must be n x n and dinv of length n");
+  double *hx = static_cast<double *>(keep_alive_alloc(sizeof(double) * (size_t)n));
+  uint64_t iters = 0;
+  double relres = 0.0;
+  {
+    DeviceMirror<int32_t> dpos(hpos, (size_t)n + 1), dcrd(hcrd, (size_t)a.nnz);
+    DeviceMirror<double> dval(hval, (size_t)a.nnz), db(hb, (size_t)n), ddinv(hdinv, (size_t)n);
+    DeviceMirror<double> dx(hx, (size_t)n, false);
+    lapis_hip_csr_plan *plan = nullptr;
+    check(lapis_hip_csr_plan_create(&plan, n, n, a.nnz, dpos.dev, dcrd.dev, 8, nullptr), "lapis_hip_csr_plan_create");
+    check(lapis_hip_pcg_f64_i32(plan, n, dpos.dev, dcrd.dev, dval.dev, db.dev, ddinv.dev, tol, (uint64_t)maxiter,
+                                dx.dev, &iters, &relres, nullptr, nullptr),
+          "lapis_hip_pcg_f64_i32");
+    lapis_hip_csr_plan_destroy(plan);
+    dx.sync_host();
+  }
+  set_result_1d(ret0, hx, n);
+  *ret1 = (size_t)iters;
+  *ret2 = relres;
+}
+
+extern "C" void py_spmm(lapis_memref_2d_f32 **ret0, lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd,
+                        lapis_memref_1d_f32 *val, const lapis_csr_specifier *spec, lapis_memref_2d_f32 *B,
+                        lapis_memref_2d_f32 *C) {
+  spmm_entry<float>(ret0, pos, crd, val, spec, B, C);
+}
+
+extern "C" void py_spmm_f64(lapis_memref_2d_f64 **ret0, lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd,
+                            lapis_memref_1d_f64 *val, const lapis_csr_specifier *spec, lapis_memref_2d_f64 *B,
+                            lapis_memref_2d_f64 *C) {
+  spmm_entry<double>(ret0, pos, crd, val, spec, B, C);
+}
+
+extern "C" void py_plus_norm(lapis_memref_1d_f64 **ret0, double *ret1, lapis_memref_1d_f64 *x,
+                             lapis_memref_1d_f64 *y) {
+  double *hx = host_data(x, 1, "x");
+  double *hy = host_data(y, 1, "y");
+  const int64_t n = y->sizes[0];  // %n = tensor.dim %y (examples/multiple_results.py:10)
+  if (x->sizes[0] < n) module_abort("plus_norm: x shorter than y");
+  double *hout = static_cast<double *>(keep_alive_alloc(sizeof(double) * (size_t)n));
+  double sum = 0.0;
+  {
+    DeviceMirror<double> dx(hx, (size_t)n), dy(hy, (size_t)n), dout(hout, (size_t)n, false);
+    double *dsum = nullptr;
+    check_hip(hipMalloc(&dsum, sizeof(double)), "hipMalloc");
+    check(lapis_hip_axpby_f64(n, 1.0, dx.dev, 1.0, dy.dev, dout.dev, nullptr), "lapis_hip_axpby_f64");
+    check(lapis_hip_dot_f64(n, dout.dev, dout.dev, 0.0, dsum, nullptr), "lapis_hip_dot_f64");
+    check_hip(hipMemcpy(&sum, dsum, sizeof(double), hipMemcpyDeviceToHost), "device-to-host copy");
+    (void)hipFree(dsum);
+    dout.sync_host();
+  }
+  set_result_1d(ret0, hout, n);
+  *ret1 = sqrt(sum);
+}

@@ -1,0 +1,694 @@
+// CSR SpMV for gfx950: the plan (row-length statistics -> kernel choice) and the
+// three kernel families it chooses from.
+//
+//   y[i] = y[i] + sum_{j in [pos[i], pos[i+1])} val[j] * x[crd[j]]
+//
+// replaces the TeamPolicy / ThreadVectorRange lambda the reference emits for
+// tests/Dialect/Kokkos/loop_mapping_2.mlir.gold:12-37.
+#include <algorithm>
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+
+#include "common.hpp"
+
+namespace lapis {
+
+// ------------------------------------------------------------------------------
+// Device helpers
+// ------------------------------------------------------------------------------
+template <bool NT, typename V>
+__device__ __forceinline__ V ld(const V *p) {
+  if (NT) return load_stream(p);
+  return *p;
+}
+
+template <bool NT>
+__device__ __forceinline__ void load4(const double *p, double (&o)[4]) {
+  v2d a = ld<NT>(reinterpret_cast<const v2d *>(p));
+  v2d b = ld<NT>(reinterpret_cast<const v2d *>(p + 2));
+  o[0] = a.x; o[1] = a.y; o[2] = b.x; o[3] = b.y;
+}
+template <bool NT>
+__device__ __forceinline__ void load4(const float *p, float (&o)[4]) {
+  v4f a = ld<NT>(reinterpret_cast<const v4f *>(p));
+  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+}
+__device__ __forceinline__ void store4_lds(double *p, const double (&v)[4]) {
+  v2d a, b;
+  a.x = v[0]; a.y = v[1]; b.x = v[2]; b.y = v[3];
+  *reinterpret_cast<v2d *>(p) = a;
+  *reinterpret_cast<v2d *>(p + 2) = b;
+}
+__device__ __forceinline__ void store4_lds(float *p, const float (&v)[4]) {
+  v4f a;
+  a.x = v[0]; a.y = v[1]; a.z = v[2]; a.w = v[3];
+  *reinterpret_cast<v4f *>(p) = a;
+}
+
+// Stage val[j]*x[crd[j]] for j in [g0, g0+count) into buf[0..count): 4 consecutive
+// non-zeros per lane, 256 per wavefront step.  `g0` is a multiple of 4 so that the
+// 128-bit loads are aligned when VEC is set; `avail` = number of array elements
+// that exist from g0 on (loads never touch anything at or beyond g0+avail).
+template <typename T, int CAP, bool VEC, bool NT>
+__device__ __forceinline__ void stage_products(T *buf, int lane, const int *__restrict__ crd,
+                                               const T *__restrict__ val, const T *__restrict__ x,
+                                               int g0, int count, int avail) {
+  constexpr int STEPS = CAP / 256;
+  if (VEC && count == CAP && avail >= CAP) {
+    // full tile: no guards, all index/value loads can be issued before the gathers
+    v4i cc[STEPS];
+    T vv[STEPS][4];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      const int k = s * 256 + lane * 4;
+      cc[s] = ld<NT>(reinterpret_cast<const v4i *>(crd + g0 + k));
+      load4<NT>(val + g0 + k, vv[s]);
+    }
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      const int k = s * 256 + lane * 4;
+      T pr[4];
+      pr[0] = vv[s][0] * x[cc[s].x];
+      pr[1] = vv[s][1] * x[cc[s].y];
+      pr[2] = vv[s][2] * x[cc[s].z];
+      pr[3] = vv[s][3] * x[cc[s].w];
+      store4_lds(buf + k, pr);
+    }
+    return;
+  }
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+    const int k = s * 256 + lane * 4;
+    if (k >= count) continue;
+    if (VEC && k + 4 <= avail) {
+      v4i c4 = ld<NT>(reinterpret_cast<const v4i *>(crd + g0 + k));
+      T v4[4], pr[4];
+      load4<NT>(val + g0 + k, v4);
+      pr[0] = v4[0] * x[c4.x];
+      pr[1] = v4[1] * x[c4.y];
+      pr[2] = v4[2] * x[c4.z];
+      pr[3] = v4[3] * x[c4.w];
+      store4_lds(buf + k, pr);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (k + e < count && k + e < avail) {
+          const int cj = ld<NT>(crd + g0 + k + e);
+          const T vj = ld<NT>(val + g0 + k + e);
+          buf[k + e] = vj * x[cj];
+        }
+      }
+    }
+  }
+}
+
+// One row piece per lane out of the staged tile: buf[lo..hi) summed in ascending
+// order by the owning lane; pieces longer than LONG_PIECE are summed by the whole
+// wavefront instead (strided partial sums + DPP reduction).
+constexpr int kLongPiece = 48;
+
+template <typename T>
+__device__ __forceinline__ T sum_piece(const T *buf, int lane, int lo, int hi) {
+  const int len = hi - lo;
+  const bool is_long = len > kLongPiece;
+  T acc = T(0);
+  if (!is_long) {
+    for (int j = lo; j < hi; ++j) acc = acc + buf[j];
+  }
+  unsigned long long m = __ballot(is_long);
+  while (m) {
+    const int src = __builtin_ctzll(m);
+    m &= m - 1;
+    const int llo = __shfl(lo, src, 64);
+    const int lhi = __shfl(hi, src, 64);
+    T part = T(0);
+    for (int j = llo + lane; j < lhi; j += 64) part = part + buf[j];
+    part = group_sum<64>(part);
+    if (lane == src) acc = part;
+  }
+  return acc;
+}
+
+// ------------------------------------------------------------------------------
+// Kernel family 1: W lanes per row
+// ------------------------------------------------------------------------------
+template <typename T, int W, bool NT>
+__global__ __launch_bounds__(256) void spmv_subwarp_kernel(int nrows, const int *__restrict__ pos,
+                                                           const int *__restrict__ crd,
+                                                           const T *__restrict__ val,
+                                                           const T *__restrict__ x, T *__restrict__ y) {
+  const long long gid = (long long)blockIdx.x * 256 + threadIdx.x;
+  const long long row = gid / W;
+  const int sub = (int)(gid % W);
+  int j = 0, end = 0;
+  if (row < nrows) {
+    j = pos[row] + sub;
+    end = pos[row + 1];
+  }
+  T acc = T(0);
+  for (; j < end; j += W) {
+    const int cj = ld<NT>(crd + j);
+    const T vj = ld<NT>(val + j);
+    acc = acc + vj * x[cj];
+  }
+  acc = group_sum<W>(acc);
+  if (sub == 0 && row < nrows) y[row] = acc + y[row];
+}
+
+// ------------------------------------------------------------------------------
+// Kernel family 2: 64 consecutive rows per wavefront, products staged in LDS
+// ------------------------------------------------------------------------------
+template <typename T, int CAP, int WAVES, bool VEC, bool NT>
+__global__ __launch_bounds__(64 * WAVES) void spmv_rowblock_kernel(
+    int nrows, int nnz, const int *__restrict__ pos, const int *__restrict__ crd,
+    const T *__restrict__ val, const T *__restrict__ x, T *__restrict__ y) {
+  __shared__ T lds[WAVES * CAP];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const long long row0 = ((long long)blockIdx.x * WAVES + wave) * 64;
+  if (row0 >= nrows) return;
+  T *buf = lds + wave * CAP;
+  const long long row = row0 + lane;
+  const bool valid = row < nrows;
+  int ps = nnz, pe = nnz;
+  if (valid) {
+    ps = pos[row];
+    pe = pos[row + 1];
+  }
+  const int base = __shfl(ps, 0, 64);
+  const int end = __shfl(pe, 63, 64);
+  T acc = T(0);
+  for (long long off = base & ~3; off < end; off += CAP) {
+    const int g0 = (int)off;
+    const int count = (int)std::min<long long>(CAP, end - off);
+    const int avail = (int)std::min<long long>(CAP, (long long)nnz - off);
+    stage_products<T, CAP, VEC, NT>(buf, lane, crd, val, x, g0, count, avail);
+    wave_lds_sync();
+    const int lo = std::max(ps, g0) - g0;
+    const int hi = (int)(std::min<long long>(pe, off + CAP) - off);
+    const T part = sum_piece(buf, lane, lo, hi);
+    acc = acc + part;
+    wave_lds_sync();
+  }
+  if (valid) y[row] = acc + y[row];
+}
+
+// ------------------------------------------------------------------------------
+// Kernel family 3: CH consecutive non-zeros per wavefront (row split)
+// ------------------------------------------------------------------------------
+// chunk_row[c] = row owning non-zero c*CH (c < nchunks), chunk_row[nchunks] = nrows.
+// A row piece that is a whole row is written to y at once; a piece of a row that
+// started in an earlier chunk goes to part_first[c], a piece of a row that
+// continues into the next chunk to part_last[c]; the fix-up kernel adds them up.
+template <typename T, int CH, int WAVES, bool VEC, bool NT>
+__global__ __launch_bounds__(64 * WAVES) void spmv_nnzsplit_kernel(
+    int nrows, int nnz, int nchunks, const int *__restrict__ pos, const int *__restrict__ crd,
+    const T *__restrict__ val, const T *__restrict__ x, T *__restrict__ y,
+    const int *__restrict__ chunk_row, T *__restrict__ part_first, T *__restrict__ part_last) {
+  __shared__ T lds[WAVES * CH];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int c = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * WAVES + wave));
+  if (c >= nchunks) return;
+  T *buf = lds + wave * CH;
+  const int e0 = c * CH;
+  const int len = std::min(CH, nnz - e0);
+  const long long e1 = (long long)e0 + len;
+  const int r0 = chunk_row[c];
+  const int r1 = std::min(chunk_row[c + 1], nrows - 1);
+
+  stage_products<T, CH, VEC, NT>(buf, lane, crd, val, x, e0, len, len);
+  wave_lds_sync();
+
+  for (long long rb = r0; rb <= r1; rb += 64) {
+    const long long r = rb + lane;
+    int ps = 0, pe = 0;
+    if (r <= r1) {
+      ps = ld<NT>(pos + r);
+      pe = ld<NT>(pos + r + 1);
+    }
+    const int lo = std::max(ps, e0) - e0;
+    const int hi = (int)(std::min<long long>(pe, e1) - e0);
+    const T acc = sum_piece(buf, lane, lo, hi);
+    if (hi > lo) {
+      const bool starts = ps >= e0;
+      const bool ends = pe <= e1;
+      if (starts && ends)
+        y[r] = acc + y[r];
+      else if (!starts)
+        part_first[c] = acc;
+      else
+        part_last[c] = acc;
+    }
+  }
+}
+
+// One thread per chunk boundary c (1 <= c < nchunks).  The row cut by boundary c
+// is completed by the thread of the FIRST boundary that cuts it:
+//   y[r] += part_last[c-1] + part_first[c] + ... + part_first[c_last]
+// in that fixed order, so the result does not depend on scheduling.
+template <typename T, int CH>
+__global__ __launch_bounds__(256) void spmv_nnzsplit_fixup_kernel(
+    int nchunks, const int *__restrict__ pos, const int *__restrict__ chunk_row,
+    const T *__restrict__ part_first, const T *__restrict__ part_last, T *__restrict__ y) {
+  const int lane = threadIdx.x & 63;
+  const long long c = (long long)blockIdx.x * 256 + threadIdx.x + 1;
+  bool owner = false;
+  int r = 0, cfirst = 0, clast = -1;
+  if (c < nchunks) {
+    r = chunk_row[c];
+    const long long ps = pos[r];
+    const long long b = c * CH;
+    if (ps < b && ps >= b - CH) {
+      owner = true;
+      cfirst = (int)c;
+      clast = (pos[r + 1] - 1) / CH;
+    }
+  }
+  const bool is_long = owner && (clast - cfirst) >= 16;
+  T total = T(0);
+  if (owner && !is_long) {
+    total = part_last[cfirst - 1];
+    for (int cc = cfirst; cc <= clast; ++cc) total = total + part_first[cc];
+  }
+  unsigned long long m = __ballot(is_long);
+  while (m) {
+    const int src = __builtin_ctzll(m);
+    m &= m - 1;
+    const int cs = __shfl(cfirst, src, 64);
+    const int cl = __shfl(clast, src, 64);
+    T part = T(0);
+    for (int cc = cs + lane; cc <= cl; cc += 64) part = part + part_first[cc];
+    part = group_sum<64>(part);
+    if (lane == src) total = part_last[cfirst - 1] + part;
+  }
+  if (owner) y[r] = total + y[r];
+}
+
+// ------------------------------------------------------------------------------
+// Plan analysis kernels
+// ------------------------------------------------------------------------------
+struct DeviceStats {
+  int min_len;
+  int max_len;
+  int bad;  // bit 0: positions decrease; bit 1: coordinate out of range
+  int pad;
+  unsigned long long empty_rows;
+  double sum_sq;
+};
+
+__global__ __launch_bounds__(256) void row_stats_kernel(int nrows, const int *__restrict__ pos,
+                                                        DeviceStats *st) {
+  const int lane = threadIdx.x & 63;
+  int mn = INT32_MAX, mx = 0, bad = 0;
+  unsigned long long empt = 0;
+  double sq = 0.0;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < nrows;
+       i += (long long)gridDim.x * 256) {
+    const int len = pos[i + 1] - pos[i];
+    if (len < 0) bad = 1;
+    mn = std::min(mn, len);
+    mx = std::max(mx, len);
+    empt += (len == 0);
+    sq += (double)len * (double)len;
+  }
+  for (int o = 32; o > 0; o >>= 1) {
+    mn = std::min(mn, __shfl_xor(mn, o, 64));
+    mx = std::max(mx, __shfl_xor(mx, o, 64));
+    bad |= __shfl_xor(bad, o, 64);
+    empt += __shfl_xor(empt, o, 64);
+    sq += __shfl_xor(sq, o, 64);
+  }
+  if (lane == 0) {
+    atomicMin(&st->min_len, mn);
+    atomicMax(&st->max_len, mx);
+    if (bad) atomicOr(&st->bad, 1);
+    if (empt) atomicAdd(&st->empty_rows, empt);
+    atomicAdd(&st->sum_sq, sq);
+  }
+}
+
+__global__ __launch_bounds__(256) void crd_range_kernel(long long nnz, int ncols,
+                                                        const int *__restrict__ crd, DeviceStats *st) {
+  int bad = 0;
+  for (long long j = (long long)blockIdx.x * 256 + threadIdx.x; j < nnz;
+       j += (long long)gridDim.x * 256) {
+    const int cj = crd[j];
+    if (cj < 0 || cj >= ncols) bad = 1;
+  }
+  if (__ballot(bad) && (threadIdx.x & 63) == 0) atomicOr(&st->bad, 2);
+}
+
+template <int CH>
+__global__ __launch_bounds__(256) void chunk_row_kernel(int nrows, int nchunks,
+                                                        const int *__restrict__ pos,
+                                                        int *__restrict__ chunk_row) {
+  const long long r = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (r == 0) chunk_row[nchunks] = nrows;
+  if (r >= nrows) return;
+  const long long ps = pos[r], pe = pos[r + 1];
+  if (pe <= ps) return;
+  const long long first = (ps + CH - 1) / CH;
+  const long long last = (pe - 1) / CH;
+  for (long long c = first; c <= last; ++c) chunk_row[c] = (int)r;
+}
+
+}  // namespace lapis
+
+// ------------------------------------------------------------------------------
+// Host side
+// ------------------------------------------------------------------------------
+using namespace lapis;
+
+namespace {
+constexpr int kChunk = 1024;      // non-zeros per wavefront in the row-split kernel
+constexpr int kRowblockCap = 1024;  // staged non-zeros per wavefront tile in the row-block kernel
+constexpr int kWavesPerBlock = 4;
+
+int env_int(const char *name, int dflt) {
+  const char *s = getenv(name);
+  return (s && *s) ? atoi(s) : dflt;
+}
+
+// LAPIS::threadParallelVectorLength (LAPISSupport.hpp:428-435) with the wave64
+// vector_length_max, including the "no hint -> 8" case (emitter :2013-2019).
+int reference_vector_length(int64_t hint) {
+  if (hint == 0) return 8;
+  int par = (int)std::min<int64_t>(hint, INT32_MAX);
+  if (par < 1) return 1;
+  int v = 1;
+  while (v < kWave && v * 6 < par) v *= 2;
+  return v;
+}
+
+int64_t reference_hint(int64_t nrows, int64_t pos_first, int64_t pos_last) {
+  if (nrows <= 0) return 0;
+  return (pos_last - pos_first + nrows - 1) / nrows;
+}
+}  // namespace
+
+struct lapis_hip_csr_plan {
+  lapis_hip_csr_stats stats;
+  const int32_t *pos;
+  int nchunks;
+  bool nontemporal;
+  int *chunk_row;     // device, int[nchunks+1]
+  void *part_first;   // device, 8 bytes * nchunks
+  void *part_last;    // device, 8 bytes * nchunks
+};
+
+namespace {
+
+void choose_kernel(lapis_hip_csr_plan *p) {
+  lapis_hip_csr_stats &s = p->stats;
+  s.chunk = 0;
+  s.width = 0;
+  if (s.nnz == 0 || s.nrows == 0) {
+    s.kernel = LAPIS_HIP_SPMV_SUBWARP;
+    s.width = 1;
+    return;
+  }
+  const double mean = s.mean_row_len;
+  const bool skewed = (double)s.max_row_len > 8.0 * std::max(mean, 32.0);
+  if (skewed || mean < 48.0) {
+    s.kernel = LAPIS_HIP_SPMV_NNZSPLIT;
+    s.chunk = kChunk;
+    return;
+  }
+  // long, even rows: enough lanes per row that a row takes about four strided steps
+  int w = 16;
+  while (w < kWave && w * 4 < mean) w *= 2;
+  s.kernel = LAPIS_HIP_SPMV_SUBWARP;
+  s.width = w;
+}
+
+template <typename T, int W, bool NT>
+int launch_subwarp_w(int64_t nrows, const int *pos, const int *crd, const T *val, const T *x, T *y,
+                     hipStream_t st) {
+  const int64_t blocks = ceil_div(nrows * W, 256);
+  if (blocks > 0x7fffffffLL)
+    return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT, "spmv: %lld rows with %d lanes per row exceed the grid limit",
+                     (long long)nrows, W);
+  launch_timed(spmv_subwarp_kernel<T, W, NT>, dim3((unsigned)blocks), dim3(256), st, (int)nrows, pos, crd, val, x,
+               y);
+  LAPIS_LAUNCH_CHECK();
+  return LAPIS_HIP_OK;
+}
+
+template <typename T, bool NT>
+int launch_subwarp(int width, int64_t nrows, const int *pos, const int *crd, const T *val, const T *x,
+                   T *y, hipStream_t st) {
+  switch (width) {
+    case 1: return launch_subwarp_w<T, 1, NT>(nrows, pos, crd, val, x, y, st);
+    case 2: return launch_subwarp_w<T, 2, NT>(nrows, pos, crd, val, x, y, st);
+    case 4: return launch_subwarp_w<T, 4, NT>(nrows, pos, crd, val, x, y, st);
+    case 8: return launch_subwarp_w<T, 8, NT>(nrows, pos, crd, val, x, y, st);
+    case 16: return launch_subwarp_w<T, 16, NT>(nrows, pos, crd, val, x, y, st);
+    case 32: return launch_subwarp_w<T, 32, NT>(nrows, pos, crd, val, x, y, st);
+    case 64: return launch_subwarp_w<T, 64, NT>(nrows, pos, crd, val, x, y, st);
+    default:
+      return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT, "spmv: lanes per row must be a power of two <= 64, got %d",
+                       width);
+  }
+}
+
+template <typename T, bool VEC, bool NT>
+int launch_rowblock(int64_t nrows, int64_t nnz, const int *pos, const int *crd, const T *val, const T *x,
+                    T *y, hipStream_t st) {
+  const int64_t blocks = ceil_div(nrows, 64 * kWavesPerBlock);
+  launch_timed(spmv_rowblock_kernel<T, kRowblockCap, kWavesPerBlock, VEC, NT>, dim3((unsigned)blocks),
+               dim3(64 * kWavesPerBlock), st, (int)nrows, (int)nnz, pos, crd, val, x, y);
+  LAPIS_LAUNCH_CHECK();
+  return LAPIS_HIP_OK;
+}
+
+template <typename T, bool VEC, bool NT>
+int launch_nnzsplit(const lapis_hip_csr_plan *p, const int *pos, const int *crd, const T *val, const T *x,
+                    T *y, hipStream_t st) {
+  const int nchunks = p->nchunks;
+  const int blocks = (int)ceil_div(nchunks, kWavesPerBlock);
+  launch_timed(spmv_nnzsplit_kernel<T, kChunk, kWavesPerBlock, VEC, NT>, dim3(blocks), dim3(64 * kWavesPerBlock),
+               st, (int)p->stats.nrows, (int)p->stats.nnz, nchunks, pos, crd, val, x, y,
+               (const int *)p->chunk_row, static_cast<T *>(p->part_first), static_cast<T *>(p->part_last));
+  LAPIS_LAUNCH_CHECK();
+  if (nchunks > 1) {
+    const int fblocks = (int)ceil_div(nchunks - 1, 256);
+    hipLaunchKernelGGL((spmv_nnzsplit_fixup_kernel<T, kChunk>), dim3(fblocks), dim3(256), 0, st, nchunks, pos,
+                       p->chunk_row, static_cast<const T *>(p->part_first),
+                       static_cast<const T *>(p->part_last), y);
+    LAPIS_LAUNCH_CHECK();
+  }
+  return LAPIS_HIP_OK;
+}
+
+template <typename T>
+int spmv_impl(lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, const int32_t *pos, const int32_t *crd,
+              const T *val, const T *x, T *y, lapis_hip_stream_t stream) {
+  LAPIS_CHECK_INIT();
+  LAPIS_REQUIRE(nrows >= 0 && ncols >= 0, "spmv: negative dimension (%lld x %lld)", (long long)nrows,
+                (long long)ncols);
+  LAPIS_REQUIRE(nrows <= INT32_MAX - 64 && ncols <= INT32_MAX, "spmv: dimensions exceed the int32 index range");
+  if (nrows == 0) return LAPIS_HIP_OK;
+  LAPIS_REQUIRE(pos && y, "spmv: null positions or output with %lld rows", (long long)nrows);
+  hipStream_t st = as_stream(stream);
+
+  if (!plan) {
+    // The reference's own rule: read pos[n] and pos[0] on the host at every call
+    // (KokkosLoopMapping.cpp:290-322), turn the mean row length into a vector length.
+    int32_t ends[2] = {0, 0};
+    LAPIS_HIP_TRY(hipMemcpyAsync(&ends[0], pos, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+    LAPIS_HIP_TRY(hipMemcpyAsync(&ends[1], pos + nrows, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+    LAPIS_HIP_TRY(hipStreamSynchronize(st));
+    const int64_t nnz = (int64_t)ends[1] - ends[0];
+    LAPIS_REQUIRE(nnz >= 0, "spmv: pos[n] < pos[0]");
+    if (nnz == 0) return LAPIS_HIP_OK;
+    LAPIS_REQUIRE(crd && val && x, "spmv: null coordinates, values or x with %lld non-zeros", (long long)nnz);
+    const int w = reference_vector_length(reference_hint(nrows, ends[0], ends[1]));
+    return launch_subwarp<T, true>(w, nrows, pos, crd, val, x, y, st);
+  }
+
+  const lapis_hip_csr_stats &s = plan->stats;
+  if (s.nrows != nrows || s.ncols != ncols || plan->pos != pos)
+    return set_error(LAPIS_HIP_ERR_PLAN_MISMATCH,
+                     "spmv: plan was built for a %lld x %lld matrix at positions %p, called with %lld x %lld at %p",
+                     (long long)s.nrows, (long long)s.ncols, (const void *)plan->pos, (long long)nrows,
+                     (long long)ncols, (const void *)pos);
+  if (s.nnz == 0) return LAPIS_HIP_OK;
+  LAPIS_REQUIRE(crd && val && x, "spmv: null coordinates, values or x with %lld non-zeros", (long long)s.nnz);
+  const bool vec = aligned16(crd) && aligned16(val);
+  const bool nt = plan->nontemporal;
+  switch (s.kernel) {
+    case LAPIS_HIP_SPMV_SUBWARP:
+      return nt ? launch_subwarp<T, true>(s.width, nrows, pos, crd, val, x, y, st)
+                : launch_subwarp<T, false>(s.width, nrows, pos, crd, val, x, y, st);
+    case LAPIS_HIP_SPMV_ROWBLOCK:
+      if (vec)
+        return nt ? launch_rowblock<T, true, true>(nrows, s.nnz, pos, crd, val, x, y, st)
+                  : launch_rowblock<T, true, false>(nrows, s.nnz, pos, crd, val, x, y, st);
+      return launch_rowblock<T, false, true>(nrows, s.nnz, pos, crd, val, x, y, st);
+    case LAPIS_HIP_SPMV_NNZSPLIT:
+      if (vec)
+        return nt ? launch_nnzsplit<T, true, true>(plan, pos, crd, val, x, y, st)
+                  : launch_nnzsplit<T, true, false>(plan, pos, crd, val, x, y, st);
+      return launch_nnzsplit<T, false, true>(plan, pos, crd, val, x, y, st);
+    default:
+      return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT, "spmv: plan holds unknown kernel %d", s.kernel);
+  }
+}
+
+void free_plan_buffers(lapis_hip_csr_plan *p) {
+  if (p->chunk_row) (void)hipFree(p->chunk_row);
+  if (p->part_first) (void)hipFree(p->part_first);
+  if (p->part_last) (void)hipFree(p->part_last);
+  p->chunk_row = nullptr;
+  p->part_first = p->part_last = nullptr;
+}
+
+}  // namespace
+
+extern "C" int lapis_hip_csr_plan_create(lapis_hip_csr_plan **out, int64_t nrows, int64_t ncols, int64_t nnz,
+                                         const int32_t *pos, const int32_t *crd, int value_bytes,
+                                         lapis_hip_stream_t stream) {
+  LAPIS_CHECK_INIT();
+  LAPIS_REQUIRE(out, "csr_plan_create: null output");
+  *out = nullptr;
+  LAPIS_REQUIRE(nrows >= 0 && ncols >= 0 && nnz >= 0, "csr_plan_create: negative size");
+  LAPIS_REQUIRE(nrows <= INT32_MAX - 64 && ncols <= INT32_MAX && nnz <= INT32_MAX,
+                "csr_plan_create: sizes exceed the int32 index range");
+  LAPIS_REQUIRE(value_bytes == 4 || value_bytes == 8, "csr_plan_create: value_bytes must be 4 or 8");
+  LAPIS_REQUIRE(pos, "csr_plan_create: null positions (a CSR matrix with n rows has n+1 positions)");
+  hipStream_t st = as_stream(stream);
+
+  int32_t ends[2] = {0, 0};
+  LAPIS_HIP_TRY(hipMemcpyAsync(&ends[0], pos, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+  LAPIS_HIP_TRY(hipMemcpyAsync(&ends[1], pos + nrows, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+  LAPIS_HIP_TRY(hipStreamSynchronize(st));
+  if (ends[0] != 0 || ends[1] != nnz)
+    return set_error(LAPIS_HIP_ERR_BAD_CSR, "csr_plan_create: pos[0]=%d pos[n]=%d, expected 0 and nnz=%lld",
+                     ends[0], ends[1], (long long)nnz);
+
+  DeviceStats init{INT32_MAX, 0, 0, 0, 0ull, 0.0};
+  DeviceStats host = init;
+  if (nrows > 0) {
+    DeviceStats *dstats = nullptr;
+    LAPIS_HIP_TRY(hipMalloc(&dstats, sizeof(DeviceStats)));
+    hipError_t e = hipMemcpyAsync(dstats, &init, sizeof(init), hipMemcpyHostToDevice, st);
+    if (e == hipSuccess) {
+      const int blocks = (int)std::min<int64_t>(ceil_div(nrows, 256), 4096);
+      hipLaunchKernelGGL(row_stats_kernel, dim3(blocks), dim3(256), 0, st, (int)nrows, pos, dstats);
+      e = hipGetLastError();
+    }
+    if (e == hipSuccess && crd && nnz > 0) {
+      const int blocks = (int)std::min<int64_t>(ceil_div(nnz, 256), 8192);
+      hipLaunchKernelGGL(crd_range_kernel, dim3(blocks), dim3(256), 0, st, (long long)nnz, (int)ncols, crd,
+                         dstats);
+      e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipMemcpyAsync(&host, dstats, sizeof(host), hipMemcpyDeviceToHost, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    (void)hipFree(dstats);
+    if (e != hipSuccess)
+      return set_error(LAPIS_HIP_ERR_RUNTIME, "csr_plan_create: analysis failed: %s", hipGetErrorString(e));
+  } else {
+    host.min_len = 0;
+  }
+  if (host.bad & 1) return set_error(LAPIS_HIP_ERR_BAD_CSR, "csr_plan_create: positions are not non-decreasing");
+  if (host.bad & 2)
+    return set_error(LAPIS_HIP_ERR_BAD_CSR, "csr_plan_create: a coordinate lies outside [0, %lld)", (long long)ncols);
+
+  lapis_hip_csr_plan *p = new lapis_hip_csr_plan();
+  memset(p, 0, sizeof(*p));
+  lapis_hip_csr_stats &s = p->stats;
+  s.nrows = nrows;
+  s.ncols = ncols;
+  s.nnz = nnz;
+  s.min_row_len = host.min_len;
+  s.max_row_len = host.max_len;
+  s.empty_rows = (int64_t)host.empty_rows;
+  s.mean_row_len = nrows ? (double)nnz / (double)nrows : 0.0;
+  s.var_row_len = nrows ? std::max(0.0, host.sum_sq / (double)nrows - s.mean_row_len * s.mean_row_len) : 0.0;
+  s.reference_hint = reference_hint(nrows, ends[0], ends[1]);
+  s.reference_vector_length = reference_vector_length(s.reference_hint);
+  p->pos = pos;
+  p->nontemporal = env_int("LAPIS_HIP_SPMV_NONTEMPORAL", 1) != 0;
+  p->nchunks = (int)ceil_div(nnz, kChunk);
+  choose_kernel(p);
+
+  // Row-split metadata is built whatever the choice, so that set_kernel can switch to it.
+  if (p->nchunks > 0) {
+    hipError_t e = hipMalloc(&p->chunk_row, sizeof(int) * ((size_t)p->nchunks + 1));
+    if (e == hipSuccess) e = hipMalloc(&p->part_first, 8 * (size_t)p->nchunks);
+    if (e == hipSuccess) e = hipMalloc(&p->part_last, 8 * (size_t)p->nchunks);
+    if (e == hipSuccess) {
+      hipLaunchKernelGGL((chunk_row_kernel<kChunk>), dim3((unsigned)ceil_div(nrows, 256)), dim3(256), 0, st,
+                         (int)nrows, p->nchunks, pos, p->chunk_row);
+      e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (e != hipSuccess) {
+      free_plan_buffers(p);
+      delete p;
+      return set_error(LAPIS_HIP_ERR_RUNTIME, "csr_plan_create: building row-split metadata failed: %s",
+                       hipGetErrorString(e));
+    }
+  }
+  *out = p;
+  return LAPIS_HIP_OK;
+}
+
+extern "C" int lapis_hip_csr_plan_set_kernel(lapis_hip_csr_plan *plan, int kernel, int width) {
+  LAPIS_REQUIRE(plan, "csr_plan_set_kernel: null plan");
+  lapis_hip_csr_stats &s = plan->stats;
+  switch (kernel) {
+    case LAPIS_HIP_SPMV_AUTO:
+      choose_kernel(plan);
+      return LAPIS_HIP_OK;
+    case LAPIS_HIP_SPMV_SUBWARP: {
+      const int w = width == 0 ? s.reference_vector_length : width;
+      LAPIS_REQUIRE(w >= 1 && w <= 64 && (w & (w - 1)) == 0,
+                    "csr_plan_set_kernel: lanes per row must be a power of two <= 64, got %d", w);
+      s.kernel = kernel;
+      s.width = w;
+      s.chunk = 0;
+      return LAPIS_HIP_OK;
+    }
+    case LAPIS_HIP_SPMV_ROWBLOCK:
+      s.kernel = kernel;
+      s.width = 0;
+      s.chunk = 0;
+      return LAPIS_HIP_OK;
+    case LAPIS_HIP_SPMV_NNZSPLIT:
+      s.kernel = kernel;
+      s.width = 0;
+      s.chunk = kChunk;
+      return LAPIS_HIP_OK;
+    default:
+      return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT, "csr_plan_set_kernel: unknown kernel %d", kernel);
+  }
+}
+
+extern "C" int lapis_hip_csr_plan_get_stats(const lapis_hip_csr_plan *plan, lapis_hip_csr_stats *stats) {
+  LAPIS_REQUIRE(plan && stats, "csr_plan_get_stats: null argument");
+  *stats = plan->stats;
+  return LAPIS_HIP_OK;
+}
+
+extern "C" int lapis_hip_csr_plan_destroy(lapis_hip_csr_plan *plan) {
+  if (!plan) return LAPIS_HIP_OK;
+  free_plan_buffers(plan);
+  delete plan;
+  return LAPIS_HIP_OK;
+}
+
+extern "C" int lapis_hip_spmv_csr_f64_i32(lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols,
+                                          const int32_t *pos, const int32_t *crd, const double *val,
+                                          const double *x, double *y, lapis_hip_stream_t stream) {
+  return spmv_impl<double>(plan, nrows, ncols, pos, crd, val, x, y, stream);
+}
+
+extern "C" int lapis_hip_spmv_csr_f32_i32(lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols,
+                                          const int32_t *pos, const int32_t *crd, const float *val,
+                                          const float *x, float *y, lapis_hip_stream_t stream) {
+  return spmv_impl<float>(plan, nrows, ncols, pos, crd, val, x, y, stream);
+}

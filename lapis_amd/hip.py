@@ -1,0 +1,260 @@
+"""ctypes binding of the C-ABI kernel library (include/lapis_hip.h).
+
+Pointers are DEVICE addresses: pass ``torch`` CUDA tensors (their ``data_ptr()`` is
+taken), or plain integers.  ``stream`` is a ``torch.cuda.Stream``, a raw
+``hipStream_t`` value, or None for torch's current stream.  The library has no CPU
+path: loading fails loudly when it has not been built.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "liblapis_hip.so")
+
+SPMV_AUTO, SPMV_SUBWARP, SPMV_ROWBLOCK, SPMV_NNZSPLIT = 0, 1, 2, 3
+KERNEL_NAMES = {SPMV_AUTO: "auto", SPMV_SUBWARP: "subwarp", SPMV_ROWBLOCK: "rowblock", SPMV_NNZSPLIT: "nnzsplit"}
+
+_i64, _u64, _vp, _int = ctypes.c_int64, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_int
+_dbl, _flt = ctypes.c_double, ctypes.c_float
+
+
+class LapisHipError(RuntimeError):
+    def __init__(self, status, name, message):
+        super().__init__("%s (%d): %s" % (name, status, message))
+        self.status = status
+        self.status_name = name
+
+
+class CsrStats(ctypes.Structure):
+    _fields_ = [("nrows", _i64), ("ncols", _i64), ("nnz", _i64),
+                ("min_row_len", _i64), ("max_row_len", _i64), ("empty_rows", _i64),
+                ("mean_row_len", _dbl), ("var_row_len", _dbl),
+                ("reference_hint", _i64), ("reference_vector_length", ctypes.c_int32),
+                ("kernel", ctypes.c_int32), ("width", ctypes.c_int32), ("chunk", ctypes.c_int32)]
+
+    def as_dict(self):
+        d = {k: getattr(self, k) for k, _ in self._fields_}
+        d["kernel_name"] = KERNEL_NAMES.get(self.kernel, "?")
+        return d
+
+
+_SIGNATURES = {
+    "lapis_hip_init": [],
+    "lapis_hip_finalize": [],
+    "lapis_hip_stream_synchronize": [_vp],
+    "lapis_hip_kernel_timing_start": [_int],
+    "lapis_hip_kernel_timing_stop": [ctypes.POINTER(_int), ctypes.POINTER(_dbl), ctypes.POINTER(_dbl),
+                                     ctypes.POINTER(_dbl)],
+    "lapis_hip_csr_plan_create": [ctypes.POINTER(_vp), _i64, _i64, _i64, _vp, _vp, _int, _vp],
+    "lapis_hip_csr_plan_set_kernel": [_vp, _int, _int],
+    "lapis_hip_csr_plan_get_stats": [_vp, ctypes.POINTER(CsrStats)],
+    "lapis_hip_csr_plan_destroy": [_vp],
+    "lapis_hip_spmv_csr_f64_i32": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp],
+    "lapis_hip_spmv_csr_f32_i32": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp],
+    "lapis_hip_spmm_csr_f32_i32": [_i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp],
+    "lapis_hip_spmm_csr_f64_i32": [_i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp],
+    "lapis_hip_dot_f64": [_i64, _vp, _vp, _dbl, _vp, _vp],
+    "lapis_hip_dot_f32": [_i64, _vp, _vp, _flt, _vp, _vp],
+    "lapis_hip_axpby_f64": [_i64, _dbl, _vp, _dbl, _vp, _vp, _vp],
+    "lapis_hip_axpby_f32": [_i64, _flt, _vp, _flt, _vp, _vp, _vp],
+    "lapis_hip_mult_f64": [_i64, _vp, _vp, _vp, _vp],
+    "lapis_hip_div_f64": [_i64, _vp, _vp, _vp, _vp],
+    "lapis_hip_fill_f64": [_i64, _dbl, _vp, _vp],
+    "lapis_hip_fill_f32": [_i64, _flt, _vp, _vp],
+    "lapis_hip_copy_f64": [_i64, _vp, _vp, _vp],
+    "lapis_hip_scale_f64": [_i64, _dbl, _vp, _vp],
+    "lapis_hip_pcg_f64_i32": [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _dbl, _u64, _vp,
+                              ctypes.POINTER(_u64), ctypes.POINTER(_dbl), _vp, _vp],
+}
+
+# every symbol include/lapis_hip.h declares
+EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + ["lapis_hip_last_error", "lapis_hip_status_name"])
+
+_lib = None
+
+
+def load(path=None):
+    """Load the kernel library (without initialising the device)."""
+    global _lib
+    if _lib is not None and path is None:
+        return _lib
+    path = path or LIB_PATH
+    if not os.path.exists(path):
+        raise FileNotFoundError("%s not found: build it first (python -m lapis_amd.build); "
+                                "there is no CPU fallback" % path)
+    lib = ctypes.CDLL(path)
+    for name, argtypes in _SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = _int
+    lib.lapis_hip_last_error.restype = ctypes.c_char_p
+    lib.lapis_hip_status_name.restype = ctypes.c_char_p
+    lib.lapis_hip_status_name.argtypes = [_int]
+    _lib = lib
+    return lib
+
+
+def check(status):
+    if status != 0:
+        lib = load()
+        raise LapisHipError(status, lib.lapis_hip_status_name(status).decode(), lib.lapis_hip_last_error().decode())
+
+
+_initialized = False
+
+
+def init():
+    """lapis_hip_init() once per process (needs a gfx950 device)."""
+    global _initialized
+    lib = load()
+    if not _initialized:
+        check(lib.lapis_hip_init())
+        _initialized = True
+    return lib
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    if isinstance(t, int):
+        return t
+    return t.data_ptr()
+
+
+def _stream(stream):
+    if stream is None:
+        import torch
+        return torch.cuda.current_stream().cuda_stream
+    if isinstance(stream, int):
+        return stream
+    return stream.cuda_stream
+
+
+def kernel_timing_start(capacity):
+    """Attach HIP event pairs to the next ``capacity`` dominant-kernel launches."""
+    check(init().lapis_hip_kernel_timing_start(capacity))
+
+
+def kernel_timing_stop():
+    """-> dict(count, mean_ms, min_ms, max_ms) of the launches timed since the start call."""
+    n, mean, mn, mx = _int(0), _dbl(0), _dbl(0), _dbl(0)
+    check(init().lapis_hip_kernel_timing_stop(ctypes.byref(n), ctypes.byref(mean), ctypes.byref(mn), ctypes.byref(mx)))
+    return {"count": n.value, "mean_ms": mean.value, "min_ms": mn.value, "max_ms": mx.value}
+
+
+class CsrPlan:
+    """Row-length statistics of one CSR matrix and the SpMV kernel chosen from them."""
+
+    def __init__(self, nrows, ncols, pos, crd, value_bytes=8, stream=None, nnz=None):
+        lib = init()
+        self._lib = lib
+        self._handle = _vp()
+        self.pos, self.crd = pos, crd  # keep the buffers alive: the plan holds pos by address
+        if nnz is None:
+            nnz = int(crd.shape[0])
+        check(lib.lapis_hip_csr_plan_create(ctypes.byref(self._handle), nrows, ncols, nnz, _ptr(pos), _ptr(crd),
+                                            value_bytes, _stream(stream)))
+
+    @property
+    def handle(self):
+        return self._handle
+
+    def stats(self):
+        s = CsrStats()
+        check(self._lib.lapis_hip_csr_plan_get_stats(self._handle, ctypes.byref(s)))
+        return s.as_dict()
+
+    def set_kernel(self, kernel, width=0):
+        check(self._lib.lapis_hip_csr_plan_set_kernel(self._handle, kernel, width))
+        return self
+
+    def destroy(self):
+        if self._handle:
+            self._lib.lapis_hip_csr_plan_destroy(self._handle)
+            self._handle = _vp()
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+def _suffix(t):
+    import torch
+    if t.dtype == torch.float64:
+        return "f64"
+    if t.dtype == torch.float32:
+        return "f32"
+    raise TypeError("values must be float32 or float64, got %s" % t.dtype)
+
+
+def spmv(plan, nrows, ncols, pos, crd, val, x, y, stream=None):
+    """y += A x.  ``plan`` may be None: the launch then follows the reference's own rule."""
+    lib = init()
+    fn = getattr(lib, "lapis_hip_spmv_csr_%s_i32" % _suffix(val))
+    check(fn(plan.handle if plan is not None else None, nrows, ncols, _ptr(pos), _ptr(crd), _ptr(val), _ptr(x),
+             _ptr(y), _stream(stream)))
+    return y
+
+
+def spmm(nrows, ncols, pos, crd, val, B, C, stream=None):
+    """C += A B with row-major B (ncols x k) and C (nrows x k)."""
+    lib = init()
+    fn = getattr(lib, "lapis_hip_spmm_csr_%s_i32" % _suffix(val))
+    k = int(C.shape[1])
+    check(fn(nrows, ncols, k, _ptr(pos), _ptr(crd), _ptr(val), _ptr(B), int(B.stride(0)), _ptr(C), int(C.stride(0)),
+             _stream(stream)))
+    return C
+
+
+def dot(x, y, result, init_value=0.0, stream=None):
+    """result[0] = init + x.y, with ``result`` a one-element device tensor (no host sync)."""
+    lib = init()
+    fn = getattr(lib, "lapis_hip_dot_%s" % _suffix(x))
+    check(fn(int(x.shape[0]), _ptr(x), _ptr(y), init_value, _ptr(result), _stream(stream)))
+    return result
+
+
+def axpby(a, x, b, y, dst, stream=None):
+    lib = init()
+    fn = getattr(lib, "lapis_hip_axpby_%s" % _suffix(x))
+    check(fn(int(x.shape[0]), a, _ptr(x), b, _ptr(y), _ptr(dst), _stream(stream)))
+    return dst
+
+
+def mult(x, y, dst, stream=None):
+    check(init().lapis_hip_mult_f64(int(x.shape[0]), _ptr(x), _ptr(y), _ptr(dst), _stream(stream)))
+    return dst
+
+
+def div(x, y, dst, stream=None):
+    check(init().lapis_hip_div_f64(int(x.shape[0]), _ptr(x), _ptr(y), _ptr(dst), _stream(stream)))
+    return dst
+
+
+def fill(dst, value, stream=None):
+    lib = init()
+    fn = getattr(lib, "lapis_hip_fill_%s" % _suffix(dst))
+    check(fn(int(dst.shape[0]), value, _ptr(dst), _stream(stream)))
+    return dst
+
+
+def copy(src, dst, stream=None):
+    check(init().lapis_hip_copy_f64(int(src.shape[0]), _ptr(src), _ptr(dst), _stream(stream)))
+    return dst
+
+
+def scale(alpha, val, stream=None):
+    check(init().lapis_hip_scale_f64(int(val.shape[0]), alpha, _ptr(val), _stream(stream)))
+    return val
+
+
+def pcg(plan, n, pos, crd, val, b, dinv, tol, maxiter, x, work=None, stream=None):
+    """CG of examples/pcg_solve.py on device buffers -> (iters, relres); x is filled in place."""
+    lib = init()
+    iters, relres = _u64(0), _dbl(0.0)
+    check(lib.lapis_hip_pcg_f64_i32(plan.handle if plan is not None else None, n, _ptr(pos), _ptr(crd), _ptr(val),
+                                    _ptr(b), _ptr(dinv), tol, maxiter, _ptr(x), ctypes.byref(iters),
+                                    ctypes.byref(relres), _ptr(work), _stream(stream)))
+    return int(iters.value), relres.value

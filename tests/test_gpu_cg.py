@@ -1,0 +1,76 @@
+"""Conjugate gradients on the GPU (device buffers, C ABI) against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import read_mtx_csr
+from gpu_util import dev
+from lapis_amd import generators as gen
+
+pytestmark = pytest.mark.gpu
+
+
+def _solve(gpu, pos, crd, val, b, dinv, tol, maxiter, with_plan=True, with_work=False):
+    n = b.shape[0]
+    dpos, dcrd = dev(pos), dev(crd)
+    plan = gpu.CsrPlan(n, n, dpos, dcrd) if with_plan else None
+    x = torch.full((n,), 7.0, dtype=torch.float64, device="cuda")
+    work = torch.empty(4 * n, dtype=torch.float64, device="cuda") if with_work else None
+    iters, relres = gpu.pcg(plan, n, dpos, dcrd, dev(val), dev(b), dev(dinv) if dinv is not None else None,
+                            tol, maxiter, x, work=work)
+    return x.cpu().numpy(), iters, relres
+
+
+def test_pcg_nos4_matches_oracle(gpu, oracle, golden):
+    g = golden["pcg_solve"]
+    pos, crd, val, shape = read_mtx_csr(g["matrix"])
+    n = shape[0]
+    import scipy.sparse as sp
+    A = sp.csr_matrix((val, crd, pos), shape=shape)
+    b = A @ np.ones(n)
+    dinv = 1.0 / A.diagonal()
+    xo, io, ro = oracle.pcg(pos, crd, val, b, dinv, g["reltol"], g["maxiter"])
+    for with_plan, with_work in ((True, False), (False, True)):
+        xg, ig, rg = _solve(gpu, pos, crd, val, b, dinv, g["reltol"], g["maxiter"], with_plan, with_work)
+        assert ig == io, "the iteration count is an index output: it must match exactly"
+        assert np.allclose(xg, xo, rtol=1e-9, atol=1e-12) and np.allclose(xg, np.ones(n), atol=1e-6)
+        assert abs(rg - ro) <= 1e-6 * ro + 1e-16
+
+
+@pytest.mark.parametrize("maxiter", [1, 2, 5, 33, 100])
+def test_unpreconditioned_fixed_iterations_on_laplace3d(gpu, oracle, maxiter):
+    A, b = gen.config5(scale=(24 / 192) ** 3)
+    xo, io, ro = oracle.pcg(A.pos, A.crd, A.val, b, np.ones(A.nrows), 0.0, maxiter)
+    xg, ig, rg = _solve(gpu, A.pos, A.crd, A.val, b, None, 0.0, maxiter)
+    assert ig == io == maxiter
+    # CG amplifies rounding differences of the dot products from iteration to iteration;
+    # 1e-12 relative per SpMV row grows to about 1e-9 on x over 100 iterations here
+    assert np.allclose(xg, xo, rtol=1e-8, atol=1e-10)
+    assert abs(rg - ro) <= 1e-7 * ro
+
+
+def test_preconditioned_equals_unpreconditioned_with_unit_dinv(gpu):
+    A, b = gen.config5(scale=(16 / 192) ** 3)
+    x1, i1, r1 = _solve(gpu, A.pos, A.crd, A.val, b, None, 1e-8, 200)
+    x2, i2, r2 = _solve(gpu, A.pos, A.crd, A.val, b, np.ones(A.nrows), 1e-8, 200)
+    assert i1 == i2 and r1 <= 1e-8
+    assert np.allclose(x1, x2, rtol=1e-10, atol=1e-14)
+
+
+def test_convergence_stops_early_and_x_is_not_touched_afterwards(gpu, oracle):
+    A, b = gen.config5(scale=(12 / 192) ** 3)
+    import scipy.sparse as sp
+    M = sp.csr_matrix((A.val, A.crd, A.pos), shape=(A.nrows, A.ncols))
+    xs = np.linspace(-1, 1, A.nrows)
+    rhs = M @ xs
+    dinv = 1.0 / M.diagonal()
+    xo, io, ro = oracle.pcg(A.pos, A.crd, A.val, rhs, dinv, 1e-10, 1000)
+    xg, ig, rg = _solve(gpu, A.pos, A.crd, A.val, rhs, dinv, 1e-10, 1000)
+    assert ig == io and ig < 1000 and rg <= 1e-10
+    assert np.allclose(xg, xs, atol=1e-7)
+    # kernels queued behind the converging iteration must leave x alone: the returned
+    # residual is the residual of the returned x
+    assert abs(np.linalg.norm(rhs - M @ xg) / np.linalg.norm(rhs) - rg) < 1e-9
+    # a huge tolerance leaves after the first update, as the reference's loop does
+    _, i1, _ = _solve(gpu, A.pos, A.crd, A.val, rhs, dinv, 1e30, 50)
+    assert i1 == 1

@@ -1,0 +1,108 @@
+"""The benchmark configurations at their full sizes on the GPU.
+
+Configs 2 and 3 (SpMV) are checked row by row against the oracle, which needs about
+a second for them; configs 4 and 5 are checked on what stays cheap at that size
+(sampled rows, a fixed-iteration prefix) and through size-independent properties:
+exact linearity under power-of-two scaling, an independent fp64 checksum computed by
+torch, and the residual identity of CG.
+"""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import TOL, assert_rows_close, dev
+from lapis_amd import generators as gen
+
+pytestmark = pytest.mark.gpu
+
+
+def _spmv_full(gpu, oracle, A, x, dtype):
+    pos, crd, val, dx = dev(A.pos), dev(A.crd), dev(A.val), dev(x)
+    want = np.zeros(A.nrows, dtype)
+    oracle.spmv(A.pos, A.crd, A.val, x, want)
+    scale = oracle.spmv_abs_scale(A.pos, A.crd, A.val, x)
+    plan = gpu.CsrPlan(A.nrows, A.ncols, pos, crd, value_bytes=np.dtype(dtype).itemsize)
+    tdt = torch.float64 if dtype == np.float64 else torch.float32
+    results = {}
+    for kid, width, name in ((0, 0, "auto"), (1, 0, "reference-width"), (2, 0, "rowblock"), (3, 0, "nnzsplit")):
+        print("full-size", name, flush=True)
+        plan.set_kernel(kid, width)
+        y = torch.zeros(A.nrows, dtype=tdt, device="cuda")
+        gpu.spmv(plan, A.nrows, A.ncols, pos, crd, val, dx, y)
+        torch.cuda.synchronize()
+        got = y.cpu().numpy()
+        assert_rows_close(got, want, scale, dtype, name)
+        results[name] = y
+    # independent checksum: sum_i y_i == sum_j val_j * x[crd_j], accumulated in fp64 by torch
+    check = (val.double() * dx.double()[crd.long()]).sum().item()
+    total_scale = float(scale.sum())
+    for name, y in results.items():
+        assert abs(y.double().sum().item() - check) <= TOL[np.dtype(dtype)] * total_scale, name
+    # linearity: scaling x by a power of two scales every product and partial sum exactly
+    plan.set_kernel(0, 0)
+    y2 = torch.zeros(A.nrows, dtype=tdt, device="cuda")
+    gpu.spmv(plan, A.nrows, A.ncols, pos, crd, val, dx * 4.0, y2)
+    torch.cuda.synchronize()
+    assert torch.equal(y2, results["auto"] * 4.0)
+    return plan.stats()
+
+
+def test_config2_spmv_fp64_full_size(gpu, oracle):
+    A, x = gen.config2()
+    assert A.nrows == 4194304
+    s = _spmv_full(gpu, oracle, A, x, np.float64)
+    assert s["reference_vector_length"] == 4 and s["nnz"] == A.nnz
+
+
+def test_config3_spmv_fp32_power_law_full_size(gpu, oracle):
+    A, x = gen.config3()
+    assert A.nrows == 2097152 and np.diff(A.pos).max() == 200000
+    _spmv_full(gpu, oracle, A, x, np.float32)
+
+
+def test_config4_spmm_fp32_full_size(gpu, oracle):
+    A, B = gen.config4()
+    k = B.shape[1]
+    pos, crd, val, dB = dev(A.pos), dev(A.crd), dev(A.val), dev(B)
+    C = torch.zeros(A.nrows, k, dtype=torch.float32, device="cuda")
+    gpu.spmm(A.nrows, A.ncols, pos, crd, val, dB, C)
+    torch.cuda.synchronize()
+    # oracle on every 97th row
+    rows = np.arange(0, A.nrows, 97)
+    sub_len = np.diff(A.pos)[rows]
+    sub_pos = np.zeros(rows.shape[0] + 1, np.int32)
+    sub_pos[1:] = np.cumsum(sub_len)
+    take = (A.pos[rows][:, None] + np.arange(32)[None, :]).ravel()
+    want = np.zeros((rows.shape[0], k), np.float32)
+    oracle.spmm(sub_pos, A.crd[take], A.val[take], B, want)
+    got = C[torch.from_numpy(rows).cuda()].cpu().numpy()
+    scale = np.abs(A.val[take]).reshape(-1, 32).astype(np.float64) @ np.ones((32, 1)) * np.abs(B).max()
+    assert np.all(np.abs(got.astype(np.float64) - want) <= 1e-5 * scale)
+    # checksum over all of C against torch's own sparse product in fp64 on a column subset
+    At = torch.sparse_csr_tensor(pos.long(), crd.long(), val.double(), size=(A.nrows, A.ncols))
+    ref = At @ dB[:, :4].double()
+    assert torch.allclose(C[:, :4].double(), ref, rtol=1e-4, atol=1e-4)
+
+
+def test_config5_cg_fp64_full_size(gpu, oracle):
+    A, b = gen.config5()
+    n = A.nrows
+    assert n == 7077888 and A.nnz == 49324032
+    pos, crd, val, db = dev(A.pos), dev(A.crd), dev(A.val), dev(b)
+    plan = gpu.CsrPlan(n, n, pos, crd)
+    x = torch.empty(n, dtype=torch.float64, device="cuda")
+    # a prefix the sequential oracle finishes in seconds
+    iters, relres = gpu.pcg(plan, n, pos, crd, val, db, None, 0.0, 10, x)
+    xo, io, ro = oracle.pcg(A.pos, A.crd, A.val, b, np.ones(n), 0.0, 10)
+    assert iters == io == 10
+    assert np.allclose(x.cpu().numpy(), xo, rtol=1e-9, atol=1e-12) and abs(relres - ro) <= 1e-9 * ro
+    # the benchmark run: exactly 100 iterations; the recurrence residual must agree with the true one
+    iters, relres = gpu.pcg(plan, n, pos, crd, val, db, None, 0.0, 100, x)
+    assert iters == 100
+    r = db.clone()
+    Ax = torch.zeros(n, dtype=torch.float64, device="cuda")
+    gpu.spmv(plan, n, n, pos, crd, val, x, Ax)
+    torch.cuda.synchronize()
+    true_relres = (torch.linalg.norm(r - Ax) / torch.linalg.norm(db)).item()
+    assert abs(true_relres - relres) <= 1e-6 * relres
+    assert relres < 0.2  # CG on the Laplacian makes steady progress

@@ -1,0 +1,128 @@
+"""The generated-module calling convention on the GPU: the reference's own example
+programs (examples/spmv_noalloc.py, spmv.py, pcg_solve.py, multiple_results.py,
+spmm_dcsr_opdsl.py) with only the module construction swapped."""
+import subprocess
+import sys
+import textwrap
+
+import numpy as np
+import pytest
+import scipy.sparse as sp
+from scipy.sparse.linalg import cg as scipy_cg
+
+from conftest import ROOT, read_mtx_csr
+from lapis_amd import generators as gen
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def module_kokkos(gpu):
+    from lapis_amd.module import LAPISModule
+    return LAPISModule()
+
+
+def test_spmv_noalloc_example(module_kokkos, golden):
+    g = golden["spmv_noalloc"]
+    rowptrs = np.array(g["pos"], dtype=np.int32)
+    colinds = np.array(g["crd"], dtype=np.int32)
+    values = np.array(g["val"], dtype=np.double)
+    m, n = g["m"], g["n"]
+    x = np.ones((n), dtype=np.double)
+    ykokkos = np.zeros((m), dtype=np.double)
+    ret = module_kokkos.spmv(rowptrs, colinds, values, ((m, n), (len(rowptrs), len(colinds), len(values))), x, ykokkos)
+    assert np.allclose(ykokkos, g["y_expected"])  # the output argument is updated in place
+    assert ret.ctypes.data == ykokkos.ctypes.data  # and the returned memref aliases it
+    # a second call accumulates: linalg.matvec adds A*x to the output
+    module_kokkos.spmv(rowptrs, colinds, values, ((m, n), (len(rowptrs), len(colinds), len(values))), x, ykokkos)
+    assert np.allclose(ykokkos, 2 * np.array(g["y_expected"]))
+
+
+def test_spmv_example_lapis_main_allocates_its_result(module_kokkos, golden):
+    g = golden["spmv_noalloc"]
+    rowptrs, colinds = np.array(g["pos"], np.int32), np.array(g["crd"], np.int32)
+    values = np.array(g["val"], np.double)
+    x = np.ones(5)
+    y1 = module_kokkos.lapis_main(rowptrs, colinds, values, ((5, 5), (6, 8, 8)), x)
+    y2 = module_kokkos.lapis_main(rowptrs, colinds, values, ((5, 5), (6, 8, 8)), 2 * x)
+    assert np.allclose(y1, g["y_expected"]) and np.allclose(y2, 2 * np.array(g["y_expected"]))
+    assert y1.ctypes.data != y2.ctypes.data  # each result stays alive until lapis_finalize
+
+
+def test_wrong_dtype_inputs_are_coerced_like_the_emitted_wrapper(module_kokkos, golden):
+    g = golden["spmv_noalloc"]
+    y = np.zeros(5)
+    module_kokkos.spmv(np.array(g["pos"], np.int64), np.array(g["crd"], np.int64), list(g["val"]),
+                       ((5, 5), (6, 8, 8)), np.ones(5, np.float64), y)
+    assert np.allclose(y, g["y_expected"])
+
+
+def test_pcg_solve_example(module_kokkos, golden, oracle):
+    g = golden["pcg_solve"]
+    pos, crd, val, shape = read_mtx_csr(g["matrix"])
+    A = sp.csr_matrix((val, crd, pos), shape=shape)
+    n, nnz = A.shape[0], A.nnz
+    xgold = np.ones((n), dtype=np.double)
+    b = A @ xgold
+    dinv = 1.0 / A.diagonal()
+    (x, numiter, relres) = module_kokkos.pcg(A.indptr, A.indices, A.data, ((n, n), (n + 1, nnz, nnz)), b, dinv,
+                                             g["reltol"], g["maxiter"])
+    [x_scipy, info] = scipy_cg(A, b, np.zeros((n)), rtol=g["reltol"], maxiter=g["maxiter"], M=np.diag(dinv))
+    assert np.allclose(x, x_scipy)
+    _, io, _ = oracle.pcg(pos, crd, val, b, dinv, g["reltol"], g["maxiter"])
+    assert int(numiter) == io and numiter.dtype == np.uint64
+
+
+def test_multiple_results_example(module_kokkos, golden):
+    g = golden["multiple_results"]
+    x, y = np.array(g["x"]), np.array(g["y"])
+    (x_plus_y, norm) = module_kokkos.plus_norm(x, y)
+    assert np.allclose(x_plus_y, x + y) and np.allclose(norm, np.linalg.norm(x + y))
+
+
+def test_spmm_example(module_kokkos, golden):
+    g = golden["spmm_dcsr"]
+    a, b = np.array(g["a_dense"]), np.array(g["b"])
+    A = sp.csr_matrix(a)
+    c = np.zeros((3, 2), np.float64)
+    module_kokkos.spmm(A.indptr, A.indices, A.data, ((3, 4), (4, A.nnz, A.nnz)), b, c)
+    assert np.allclose(c, np.matmul(a, b))
+
+
+def test_module_spmv_on_benchmark_shaped_input(module_kokkos, oracle):
+    A, x = gen.config2(scale=1 / 128)
+    y = np.zeros(A.nrows)
+    module_kokkos.spmv(A.pos, A.crd, A.val, A.spec(), x, y)
+    want = np.zeros(A.nrows)
+    oracle.spmv(A.pos, A.crd, A.val, x, want)
+    scale = oracle.spmv_abs_scale(A.pos, A.crd, A.val, x)
+    assert np.all(np.abs(y - want) <= 1e-12 * np.maximum(scale, 1e-300))
+    B, xf = gen.config3(scale=1 / 64)
+    yf = np.zeros(B.nrows, np.float32)
+    module_kokkos.spmv(B.pos, B.crd, B.val, B.spec(), xf, yf)
+    wantf = np.zeros(B.nrows, np.float32)
+    oracle.spmv(B.pos, B.crd, B.val, xf, wantf)
+    scalef = oracle.spmv_abs_scale(B.pos, B.crd, B.val, xf)
+    assert np.all(np.abs(yf.astype(np.float64) - wantf) <= 1e-5 * np.maximum(scalef, 1e-300))
+
+
+def test_non_contiguous_memref_aborts_like_kokkos_abort():
+    # the reference aborts the process (LAPISSupport.hpp:76,86); run it in a child
+    code = textwrap.dedent("""
+        import ctypes, numpy as np, sys
+        sys.path.insert(0, %r)
+        from lapis_amd.module import LAPISModule
+        from lapis_amd import memref as rt
+        m = LAPISModule()
+        pos = np.array([0, 1, 2], np.int32); crd = np.array([0, 1], np.int32); val = np.ones(2)
+        x2 = np.ones(4)[::2]          # stride 2: numpy.require(..., 'C') would copy, so call the C entry directly
+        y = np.zeros(2)
+        spec = np.array([2, 2, 3, 2, 2], np.int64)
+        ret0 = ctypes.pointer(ctypes.pointer(rt.make_nd_memref_descriptor(1, ctypes.c_double)()))
+        d = lambda a: ctypes.pointer(rt.get_ranked_memref_descriptor(a))
+        m.libHandle.py_spmv(ret0, d(pos), d(crd), d(val), spec.ctypes.data_as(ctypes.c_void_p), d(x2), d(y))
+        print("survived")
+    """ % ROOT)
+    proc = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert proc.returncode != 0 and "survived" not in proc.stdout
+    assert "not contiguous" in proc.stderr

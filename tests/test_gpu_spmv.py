@@ -1,0 +1,169 @@
+"""SpMV parity on the GPU: every kernel family of the HIP library, called through the
+C ABI, against the sequential-order CPU oracle on the same seeded inputs."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import assert_rows_close, dev, dev_unaligned, from_lengths as _from_lengths
+from lapis_amd import generators as gen
+from lapis_amd.generators import CSR
+
+pytestmark = pytest.mark.gpu
+
+# (kernel, width) choices a plan can be forced to, plus None = automatic choice
+KERNELS = [("auto", 0), ("subwarp", 1), ("subwarp", 2), ("subwarp", 4), ("subwarp", 8), ("subwarp", 16),
+           ("subwarp", 32), ("subwarp", 64), ("rowblock", 0), ("nnzsplit", 0)]
+KID = {"auto": 0, "subwarp": 1, "rowblock": 2, "nnzsplit": 3}
+
+
+def _matrices(dtype):
+    """name -> CSR.  Sizes are chosen so the oracle needs well under a second each."""
+    out = {}
+    out["golden5x5"] = CSR(5, 5, np.array([0, 1, 5, 6, 8, 8], np.int32),
+                           np.array([1, 0, 2, 3, 4, 2, 0, 1], np.int32),
+                           np.array([1.1, 0.3, 2.2, 3.7, -4, -19, -2, 1], dtype))
+    A, _ = gen.config1(scale=1 / 16)
+    out["laplace2d_64"] = CSR(A.nrows, A.ncols, A.pos, A.crd, A.val.astype(dtype))
+    A, _ = gen.config5(scale=(20 / 192) ** 3)
+    out["laplace3d_20"] = CSR(A.nrows, A.ncols, A.pos, A.crd, A.val.astype(dtype))
+    A = gen.poisson_random(65536 + 37, 16.0, seed=2002, dtype=dtype)
+    out["poisson16_65573"] = A
+    A = gen.powerlaw_random(131072, 30.0, 200000, seed=3003, dtype=dtype)
+    out["powerlaw_131072"] = A
+    # ragged edge cases
+    out["all_rows_empty"] = _from_lengths([0] * 300, 300, 1, dtype)
+    out["one_long_row"] = _from_lengths([5000], 8000, 2, dtype)
+    out["long_rows_between_empties"] = _from_lengths([0, 0, 3000, 0, 1, 0, 2047, 1025, 0, 0, 1, 4096, 0], 5000, 3, dtype)
+    out["chunk_boundary_exact"] = _from_lengths([1024, 1024, 512, 512, 1, 1023, 2048], 4096, 4, dtype)
+    out["wide_gap_of_empty_rows"] = _from_lengths([7] * 10 + [0] * 1000 + [9] * 10, 64, 5, dtype)
+    out["dense_short"] = _from_lengths([64] * 257, 64, 6, dtype)
+    out["mean_100"] = gen.poisson_random(3000, 100.0, seed=7, dtype=dtype)
+    return out
+
+
+@pytest.fixture(scope="module", params=[np.float64, np.float32], ids=["f64", "f32"])
+def cases(request, oracle):
+    dtype = request.param
+    built = {}
+    for name, A in _matrices(dtype).items():
+        x = gen.uniform_vector(A.ncols, 11, dtype=dtype)
+        y_in = gen.uniform_vector(A.nrows, 12, dtype=dtype)
+        want = y_in.copy()
+        oracle.spmv(A.pos, A.crd, A.val, x, want)
+        scale = oracle.spmv_abs_scale(A.pos, A.crd, A.val, x, y_in)
+        built[name] = (A, x, y_in, want, scale)
+    return dtype, built
+
+
+@pytest.mark.parametrize("kernel,width", KERNELS, ids=["%s%s" % (k, w or "") for k, w in KERNELS])
+def test_spmv_matches_oracle(gpu, cases, kernel, width):
+    dtype, built = cases
+    for name, (A, x, y_in, want, scale) in built.items():
+        print("case", name, kernel, width, np.dtype(dtype).name, flush=True)
+        pos, crd, val = dev(A.pos), dev(A.crd), dev(A.val)
+        plan = gpu.CsrPlan(A.nrows, A.ncols, pos, crd, value_bytes=np.dtype(dtype).itemsize)
+        if kernel != "auto":
+            plan.set_kernel(KID[kernel], width)
+        y = dev(y_in)
+        gpu.spmv(plan, A.nrows, A.ncols, pos, crd, val, dev(x), y)
+        torch.cuda.synchronize()
+        got = y.cpu().numpy()
+        assert_rows_close(got, want, scale, dtype, "%s/%s%d" % (name, kernel, width))
+        if kernel == "subwarp" and width == 1:
+            # one lane per row sums in the reference's order with separate multiply and add
+            assert np.array_equal(got, want), name + ": thread-per-row must be bit-identical to the oracle"
+        plan.destroy()
+
+
+def test_spmv_without_plan_follows_the_reference_rule(gpu, cases):
+    dtype, built = cases
+    for name, (A, x, y_in, want, scale) in built.items():
+        print("case", name, "no plan", flush=True)
+        y = dev(y_in)
+        gpu.spmv(None, A.nrows, A.ncols, dev(A.pos), dev(A.crd), dev(A.val), dev(x), y)
+        torch.cuda.synchronize()
+        assert_rows_close(y.cpu().numpy(), want, scale, dtype, name + "/noplan")
+
+
+def test_plan_statistics_and_reference_decision(gpu, oracle):
+    A, _ = gen.config2(scale=1 / 64)
+    pos, crd = dev(A.pos), dev(A.crd)
+    s = gpu.CsrPlan(A.nrows, A.ncols, pos, crd).stats()
+    L = np.diff(A.pos)
+    assert (s["nrows"], s["ncols"], s["nnz"]) == (A.nrows, A.ncols, A.nnz)
+    assert (s["min_row_len"], s["max_row_len"], s["empty_rows"]) == (L.min(), L.max(), int((L == 0).sum()))
+    assert abs(s["mean_row_len"] - L.mean()) < 1e-12 and abs(s["var_row_len"] - L.var()) < 1e-6
+    # index outputs are bit-exact: the reference's hint and vector length for this matrix
+    assert s["reference_hint"] == oracle.csr_parallelism_hint(A.pos) == 16
+    assert s["reference_vector_length"] == oracle.thread_parallel_vector_length(16, 64) == 4
+    assert s["kernel_name"] == "nnzsplit"
+    B, _ = gen.config3(scale=1 / 16)
+    sb = gpu.CsrPlan(B.nrows, B.ncols, dev(B.pos), dev(B.crd), value_bytes=4).stats()
+    assert sb["kernel_name"] == "nnzsplit" and sb["reference_vector_length"] == 8
+    C = gen.poisson_random(2000, 300.0, seed=3)
+    sc = gpu.CsrPlan(C.nrows, C.ncols, dev(C.pos), dev(C.crd)).stats()
+    assert sc["kernel_name"] == "subwarp" and sc["width"] == 64
+
+
+def test_unaligned_buffers_take_the_scalar_path(gpu, oracle):
+    A = gen.poisson_random(5000, 20.0, seed=9)
+    x = gen.uniform_vector(A.ncols, 1)
+    want = np.zeros(A.nrows)
+    oracle.spmv(A.pos, A.crd, A.val, x, want)
+    scale = oracle.spmv_abs_scale(A.pos, A.crd, A.val, x)
+    pos, crd, val = dev(A.pos), dev_unaligned(A.crd), dev_unaligned(A.val)
+    for kid in (2, 3):
+        plan = gpu.CsrPlan(A.nrows, A.ncols, pos, crd).set_kernel(kid)
+        y = torch.zeros(A.nrows, dtype=torch.float64, device="cuda")
+        gpu.spmv(plan, A.nrows, A.ncols, pos, crd, val, dev(x), y)
+        torch.cuda.synchronize()
+        assert_rows_close(y.cpu().numpy(), want, scale, np.float64, "unaligned/%d" % kid)
+
+
+def test_repeated_calls_accumulate_and_are_deterministic(gpu, oracle):
+    A = gen.powerlaw_random(20000, 30.0, 200000, seed=5, dtype=np.float64)
+    x = gen.uniform_vector(A.ncols, 2)
+    pos, crd, val, dx = dev(A.pos), dev(A.crd), dev(A.val), dev(x)
+    plan = gpu.CsrPlan(A.nrows, A.ncols, pos, crd)
+    runs = []
+    for _ in range(2):
+        y = torch.zeros(A.nrows, dtype=torch.float64, device="cuda")
+        for _ in range(3):
+            gpu.spmv(plan, A.nrows, A.ncols, pos, crd, val, dx, y)
+        torch.cuda.synchronize()
+        runs.append(y.cpu().numpy())
+    assert np.array_equal(runs[0], runs[1])  # fixed summation order, no atomics on y
+    want = np.zeros(A.nrows)
+    for _ in range(3):
+        oracle.spmv(A.pos, A.crd, A.val, x, want)
+    assert_rows_close(runs[0], want, 3 * oracle.spmv_abs_scale(A.pos, A.crd, A.val, x), np.float64, "3 calls")
+
+
+def test_bad_structure_is_rejected_before_any_kernel_reads_it(gpu):
+    pos = dev(np.array([0, 2, 1, 3], np.int32))
+    crd = dev(np.array([0, 1, 2], np.int32))
+    with pytest.raises(gpu.LapisHipError) as e:
+        gpu.CsrPlan(3, 3, pos, crd)
+    assert e.value.status_name == "LAPIS_HIP_ERR_BAD_CSR"
+    pos = dev(np.array([0, 1, 2, 3], np.int32))
+    with pytest.raises(gpu.LapisHipError) as e:
+        gpu.CsrPlan(3, 3, pos, dev(np.array([0, 3, 1], np.int32)))
+    assert e.value.status_name == "LAPIS_HIP_ERR_BAD_CSR"
+    with pytest.raises(gpu.LapisHipError) as e:
+        gpu.CsrPlan(3, 3, pos, crd, nnz=5)
+    assert e.value.status_name == "LAPIS_HIP_ERR_BAD_CSR"
+    plan = gpu.CsrPlan(3, 3, pos, crd)
+    other = dev(np.array([0, 1, 2, 3], np.int32))
+    y = torch.zeros(3, dtype=torch.float64, device="cuda")
+    with pytest.raises(gpu.LapisHipError) as e:
+        gpu.spmv(plan, 3, 3, other, crd, y, y, y)
+    assert e.value.status_name == "LAPIS_HIP_ERR_PLAN_MISMATCH"
+
+
+def test_empty_matrix_is_a_no_op(gpu):
+    pos = dev(np.zeros(1, np.int32))
+    crd = torch.empty(0, dtype=torch.int32, device="cuda")
+    plan = gpu.CsrPlan(0, 0, pos, crd)
+    y = torch.empty(0, dtype=torch.float64, device="cuda")
+    gpu.spmv(plan, 0, 0, pos, crd, y, y, y)
+    torch.cuda.synchronize()
