@@ -240,6 +240,9 @@ def main():
                     help="force an SpMV kernel family instead of the plan's choice")
     ap.add_argument("--width", type=int, default=0, help="lanes per row with --kernel subwarp (0 = the reference's rule)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch the library's copy kernel on 1 GiB three times, the known-size reference "
+                         "that rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -250,6 +253,14 @@ def main():
     import torch
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU: the HIP library has no CPU path")
+    if args.calibrate_copy:
+        from lapis_amd import hip
+        src = torch.ones(1 << 27, dtype=torch.float64, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            hip.copy(src, dst)
+        torch.cuda.synchronize()
+        del src, dst
     if args.config in (1, 2, 3):
         out = run_spmv(args, args.config)
     elif args.config == 4:

@@ -45,7 +45,12 @@ def get_ranked_memref_descriptor(array):
 
 
 def ranked_memref_to_numpy(desc):
-    """numpy view aliasing the memory a descriptor points at (no copy, no ownership)."""
+    """numpy view aliasing the memory a descriptor points at (no copy, no ownership).
+
+    Takes a pointer to a descriptor, as the emitted wrappers pass it (``ret0[0]``), or
+    the descriptor itself."""
+    if not hasattr(desc, "aligned"):
+        desc = desc[0]
     rank = len(desc.shape) if hasattr(desc, "shape") else 0
     shape = tuple(desc.shape) if rank else ()
     ctype = type(desc.aligned.contents) if bool(desc.aligned) else desc._fields_[1][1]._type_
