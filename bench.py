@@ -65,7 +65,16 @@ def run_spmv(args, cfg):
     import torch
     from lapis_amd import generators as gen
     from lapis_amd import hip
+    if args.workload:
+        maker0, t_mi300a, t_h100 = gen.PUBLISHED[args.workload]
+        published = {"matrix": args.workload, "MI300A_s": t_mi300a, "H100_s": t_h100,
+                     "source": "benchmarks/plots/spmv.csv of the reference (mean of 1000 fenced calls)"}
+        cfg = 0
+    else:
+        published = None
     name, maker, dtype = {
+        0: ("%s (structure of the reference's published matrix), SpMV fp64" % args.workload,
+            (lambda: (maker0(), None)) if args.workload else None, np.float64),
         1: ("config1: SpMV fp64, 2-D 5-point Laplacian 256x256", gen.config1, np.float64),
         2: ("config2: SpMV fp64, n=4194304, Poisson(16) rows, uniform random sorted columns, int32 indices",
             gen.config2, np.float64),
@@ -74,6 +83,8 @@ def run_spmv(args, cfg):
     }[cfg]
     t0 = time.perf_counter()
     A, x = maker()
+    if x is None:
+        x = gen.uniform_vector(A.ncols, 77)
     log("generated %s: %d rows, %d nnz in %.1f s" % (name, A.nrows, A.nnz, time.perf_counter() - t0))
     dev = lambda a: torch.from_numpy(a).cuda()
     pos, crd, val, dx = dev(A.pos), dev(A.crd), dev(A.val), dev(x)
@@ -82,7 +93,13 @@ def run_spmv(args, cfg):
     plan = hip.CsrPlan(A.nrows, A.ncols, pos, crd, value_bytes=np.dtype(dtype).itemsize)
     torch.cuda.synchronize()
     plan_ms = (time.perf_counter() - t0) * 1e3
-    if args.kernel:
+    build_ms = None
+    if args.kernel == "colblock" or (args.kernel is None and plan.stats()["colblock_recommended"]):
+        t0 = time.perf_counter()
+        plan.build_colblock(crd, val)
+        torch.cuda.synchronize()
+        build_ms = (time.perf_counter() - t0) * 1e3
+    elif args.kernel:
         plan.set_kernel({"subwarp": 1, "rowblock": 2, "nnzsplit": 3}[args.kernel], args.width)
     stats = plan.stats()
     for _ in range(args.warmup):
@@ -105,7 +122,8 @@ def run_spmv(args, cfg):
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f64" if dtype == np.float64 else "f32", "data": "synthetic",
-        "config": {"workload": name, "nrows": A.nrows, "nnz": A.nnz, "seed": {1: 1001, 2: 2002, 3: 3003}[cfg],
+        "config": {"workload": name, "nrows": A.nrows, "nnz": A.nnz, "seed": {0: 77, 1: 1001, 2: 2002, 3: 3003}[cfg],
+                   "colblock_build_ms": build_ms, "mean_chunk_col_span": stats["mean_chunk_col_span"],
                    "algorithmic_bytes_per_step": bytes_step, "kernel": stats["kernel_name"],
                    "width": stats["width"], "chunk": stats["chunk"],
                    "reference_vector_length": stats["reference_vector_length"], "plan_ms": plan_ms},
@@ -113,9 +131,20 @@ def run_spmv(args, cfg):
         "gflops": 2.0 * A.nnz / (ms * 1e-3) / 1e9,
         "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": traffic_from_profiles("%s_config%d" % (stats["kernel_name"], cfg)),
+                     "traffic": traffic_from_profiles("%s_config%d" % (stats["kernel_name"], cfg)) if cfg else None,
                      "kernel_ms_mean": kt["mean_ms"], "kernel_ms_min": kt["min_ms"], "launches_timed": kt["count"]},
     }
+    if published:
+        # fenced per-call protocol of the published numbers: one call, one synchronise
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            hip.spmv(plan, A.nrows, A.ncols, pos, crd, val, dx, y)
+            torch.cuda.synchronize()
+        fenced = (time.perf_counter() - t0) / args.steps
+        published["this_run_fenced_s"] = fenced
+        published["speedup_vs_MI300A"] = published["MI300A_s"] / fenced
+        published["speedup_vs_H100"] = published["H100_s"] / fenced
+        out["published_comparison"] = published
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_spmv(A, x)
     return out
@@ -236,7 +265,9 @@ def main():
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5])
-    ap.add_argument("--kernel", choices=["subwarp", "rowblock", "nnzsplit"], default=None,
+    ap.add_argument("--workload", choices=["Laplace3D_100", "Elasticity3D_60"], default=None,
+                    help="SpMV on the structure of one of the reference's published matrices instead of a config")
+    ap.add_argument("--kernel", choices=["subwarp", "rowblock", "nnzsplit", "colblock"], default=None,
                     help="force an SpMV kernel family instead of the plan's choice")
     ap.add_argument("--width", type=int, default=0, help="lanes per row with --kernel subwarp (0 = the reference's rule)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -246,6 +277,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+    if args.workload:
+        args.config = 1  # takes the SpMV path; run_spmv swaps the matrix in
     if args.steps is None:
         args.steps = {1: 1000, 2: 200, 3: 200, 4: 20, 5: 100}[args.config]
     if args.warmup is None:

@@ -74,13 +74,18 @@ enum lapis_hip_spmv_kernel {
   LAPIS_HIP_SPMV_ROWBLOCK = 2,
   /* equal non-zero count per wavefront whatever the row lengths (row split);
    * rows cut by a chunk boundary are completed by a small second kernel. */
-  LAPIS_HIP_SPMV_NNZSPLIT = 3
+  LAPIS_HIP_SPMV_NNZSPLIT = 3,
+  /* column-blocked copy of the matrix, see lapis_hip_csr_plan_build_colblock */
+  LAPIS_HIP_SPMV_COLBLOCK = 4
 };
 
 typedef struct lapis_hip_csr_stats {
   int64_t nrows, ncols, nnz;
   int64_t min_row_len, max_row_len, empty_rows;
   double mean_row_len, var_row_len;
+  /* mean over chunks of 1024 consecutive non-zeros of (max column - min column):
+   * how far the gathers of one wavefront wander over x; -1 if crd was not given */
+  double mean_chunk_col_span;
   /* the reference's own decision for this matrix, for comparison:
    * hint = ceil((pos[n]-pos[0])/n) (KokkosLoopMapping.cpp:279-323) and
    * LAPIS::threadParallelVectorLength(hint) with vector_length_max = 64
@@ -91,6 +96,11 @@ typedef struct lapis_hip_csr_stats {
   int32_t kernel;      /* enum lapis_hip_spmv_kernel, never AUTO */
   int32_t width;       /* lanes per row for SUBWARP, else 0 */
   int32_t chunk;       /* non-zeros per wavefront for NNZSPLIT, else 0 */
+  /* 1 if lapis_hip_csr_plan_build_colblock is expected to pay for this matrix (x far
+   * larger than an XCD's L2, gathers spread all over it, even rows); plan creation
+   * cannot build it itself because it is not given the values */
+  int32_t colblock_recommended;
+  int32_t reserved;
 } lapis_hip_csr_stats;
 
 typedef struct lapis_hip_csr_plan lapis_hip_csr_plan;
@@ -110,6 +120,18 @@ int lapis_hip_csr_plan_create(lapis_hip_csr_plan **plan, int64_t nrows, int64_t 
  * (0 = the reference's rule); other kernels ignore it. */
 int lapis_hip_csr_plan_set_kernel(lapis_hip_csr_plan *plan, int kernel, int width);
 int lapis_hip_csr_plan_get_stats(const lapis_hip_csr_plan *plan, lapis_hip_csr_stats *stats);
+/* Opt-in layout for matrices whose x does not fit the 4 MB L2 of an XCD (wide,
+ * uniformly random columns): copies crd/val once into an order in which each
+ * wavefront owns 1024 consecutive rows and walks their non-zeros slice by slice of
+ * x (2^slice_log2_cols columns per slice, 0 = 1 MB of x), so that the whole chip
+ * gathers from the same few slices at a time and they stay in L2.  Same 4+sizeof(T)
+ * bytes per non-zero as CSR.  The reference has no counterpart (its launch never
+ * looks at columns, KokkosLoopMapping.cpp:861-862).  Needs
+ * ceil(log2(ncols)) <= 22.  The copy holds the VALUES as they are now: build again
+ * after changing val.  Selects the COLBLOCK kernel on success; SpMV calls with this
+ * plan then ignore their crd/val arguments.  Synchronises `stream`. */
+int lapis_hip_csr_plan_build_colblock(lapis_hip_csr_plan *plan, const int32_t *crd, const void *val,
+                                      int value_bytes, int slice_log2_cols, lapis_hip_stream_t stream);
 int lapis_hip_csr_plan_destroy(lapis_hip_csr_plan *plan);
 
 /* ---- SpMV ------------------------------------------------------------------ */

@@ -4,6 +4,7 @@ Outputs (in-tree, next to this package, so that they travel with a source snapsh
     lapis_amd/lib/liblapis_hip.so             the C-ABI kernel library (include/lapis_hip.h)
     lapis_amd/lib/liblapis_package_module.so  lapis_initialize / lapis_finalize / py_<func>
                                               (include/lapis_module.h), linked against the former
+    lapis_amd/bin/lapis_spmv_bench            MatrixMarket SpMV benchmark driver (csrc/spmv_bench_main.cpp)
 
 hipcc cross-compiles without a GPU.  Run ``python -m lapis_amd.build``.
 """
@@ -20,11 +21,13 @@ LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(CSRC, "build")
 INCLUDE = os.path.join(ROOT, "include")
 
-KERNEL_SOURCES = ["runtime.hip", "spmv.hip", "spmm.hip", "blas1.hip", "cg.hip"]
+KERNEL_SOURCES = ["runtime.hip", "spmv.hip", "colblock.hip", "spmm.hip", "blas1.hip", "cg.hip"]
 SHIM_SOURCES = ["module_shim.hip"]
 
 KERNEL_LIB = os.path.join(LIBDIR, "liblapis_hip.so")
 MODULE_LIB = os.path.join(LIBDIR, "liblapis_package_module.so")
+BINDIR = os.path.join(HERE, "bin")
+BENCH_BIN = os.path.join(BINDIR, "lapis_spmv_bench")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -73,9 +76,14 @@ def build(verbose=False, jobs=8):
     _run([_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *kobjs, "-o", KERNEL_LIB])
     _run([_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *sobjs, "-L", LIBDIR, "-llapis_hip",
           "-Wl,-rpath,$ORIGIN", "-o", MODULE_LIB])
+    os.makedirs(BINDIR, exist_ok=True)
+    _run([_hipcc(), "--offload-arch=gfx950", "-O2", "-std=c++17", "-I", INCLUDE,
+          os.path.join(CSRC, "spmv_bench_main.cpp"), "-L", LIBDIR, "-llapis_hip", "-Wl,-rpath,$ORIGIN/../lib", "-o",
+          BENCH_BIN])
     if verbose:
         print("built", KERNEL_LIB)
         print("built", MODULE_LIB)
+        print("built", BENCH_BIN)
     return KERNEL_LIB, MODULE_LIB
 
 

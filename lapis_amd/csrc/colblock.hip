@@ -1,0 +1,427 @@
+// Column-blocked SpMV: the variant for matrices whose gathered vector x does not
+// fit the 4 MB L2 of an XCD (uniformly random columns over millions of columns).
+//
+// A gather that misses L2 pulls a 128-byte line for 8 useful bytes, so the plain
+// CSR kernels spend the HBM bandwidth on line fills.  Here the matrix is copied
+// once, at plan time, into an order in which every wavefront owns 1024 consecutive
+// rows and walks their non-zeros slice by slice of x (slice = 2^s consecutive
+// columns, 1 MB of x by default).  All wavefronts are resident at once and start
+// together, so at any moment the whole chip is gathering from the same few slices
+// and they stay in L2.  Row sums are accumulated in LDS (one accumulator per row
+// of the wave's block) and written to y once.
+//
+// Entry format: one uint32 = (row within the block << col_bits) | column, plus the
+// value; 12 bytes per non-zero for fp64, exactly the CSR footprint, and `pos` is
+// only read at row-block boundaries.
+#include <hipcub/hipcub.hpp>
+
+#include <algorithm>
+#include <cstdlib>
+
+#include "common.hpp"
+#include "plan.hpp"
+
+namespace lapis {
+
+template <bool NT, typename V>
+__device__ __forceinline__ V ldv(const V *p) {
+  if (NT) return load_stream(p);
+  return *p;
+}
+
+__device__ __forceinline__ void lds_add(double *p, double v) { unsafeAtomicAdd(p, v); }
+__device__ __forceinline__ void lds_add(float *p, float v) { unsafeAtomicAdd(p, v); }
+
+template <bool NT>
+__device__ __forceinline__ void load4v(const double *p, double (&o)[4]) {
+  v2d a = ldv<NT>(reinterpret_cast<const v2d *>(p));
+  v2d b = ldv<NT>(reinterpret_cast<const v2d *>(p + 2));
+  o[0] = a.x; o[1] = a.y; o[2] = b.x; o[3] = b.y;
+}
+template <bool NT>
+__device__ __forceinline__ void load4v(const float *p, float (&o)[4]) {
+  v4f a = ldv<NT>(reinterpret_cast<const v4f *>(p));
+  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+}
+
+// One wavefront per block of RB rows.  STEPS * 256 entries are in flight per loop trip.
+// Loads EPL consecutive entries (index words and values) for one lane.
+template <bool NT>
+__device__ __forceinline__ void load_entries(const unsigned *bi, const double *bv, long long p, unsigned (&i)[4],
+                                             double (&v)[4]) {
+  v4i c = ldv<NT>(reinterpret_cast<const v4i *>(bi + p));
+  i[0] = (unsigned)c.x; i[1] = (unsigned)c.y; i[2] = (unsigned)c.z; i[3] = (unsigned)c.w;
+  load4v<NT>(bv + p, v);
+}
+template <bool NT>
+__device__ __forceinline__ void load_entries(const unsigned *bi, const float *bv, long long p, unsigned (&i)[4],
+                                             float (&v)[4]) {
+  v4i c = ldv<NT>(reinterpret_cast<const v4i *>(bi + p));
+  i[0] = (unsigned)c.x; i[1] = (unsigned)c.y; i[2] = (unsigned)c.z; i[3] = (unsigned)c.w;
+  load4v<NT>(bv + p, v);
+}
+template <bool NT, typename T>
+__device__ __forceinline__ void load_entries(const unsigned *bi, const T *bv, long long p, unsigned (&i)[2], T (&v)[2]) {
+  v2i c = ldv<NT>(reinterpret_cast<const v2i *>(bi + p));
+  i[0] = (unsigned)c.x; i[1] = (unsigned)c.y;
+  v[0] = ldv<NT>(bv + p);
+  v[1] = ldv<NT>(bv + p + 1);
+}
+template <bool NT, typename T>
+__device__ __forceinline__ void load_entries(const unsigned *bi, const T *bv, long long p, unsigned (&i)[1], T (&v)[1]) {
+  i[0] = ldv<NT>(bi + p);
+  v[0] = ldv<NT>(bv + p);
+}
+
+// One wavefront per block of RB rows.  A trip handles STEPS * 64 * EPL entries; the
+// index words and values of the NEXT trip are already in flight while this trip's
+// gathers run, so the streamed arrays keep many loads outstanding while the window
+// of x a wavefront is gathering from stays small.  PAD ints of unused LDS per
+// workgroup set how many workgroups fit a CU (an even spread keeps the wavefronts
+// of the chip moving through x at the same pace).
+template <typename T, int RB, int WAVES, int STEPS, int EPL, int PAD, bool NT>
+__global__ __launch_bounds__(64 * WAVES) void spmv_colblock_kernel(int nrows, int nnz, int col_bits,
+                                                                   const int *__restrict__ pos,
+                                                                   const unsigned *__restrict__ bidx,
+                                                                   const T *__restrict__ bval,
+                                                                   const T *__restrict__ x, T *__restrict__ y,
+                                                                   unsigned pace_fp) {
+  __shared__ T lds[WAVES * RB + PAD];
+  const long long t0 = wall_clock64();
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int rb = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * WAVES + wave));
+  const long long row0 = (long long)rb * RB;
+  if (row0 >= nrows) return;
+  const int rows_here = (int)std::min<long long>(RB, nrows - row0);
+  T *acc = lds + wave * RB;
+  if (PAD > 0 && nrows < 0) lds[WAVES * RB + lane] = T(0);  // keeps the padding allocated
+#pragma unroll
+  for (int i = 0; i < RB / 64; ++i) acc[i * 64 + lane] = T(0);
+  wave_lds_sync();
+
+  const int start = pos[row0];
+  const int end = pos[row0 + rows_here];
+  const unsigned col_mask = (1u << col_bits) - 1u;
+  constexpr int STEP = 64 * EPL;
+  constexpr int TRIP = STEPS * STEP;
+  const long long first = start & ~3;
+  // entries of one trip, guarded: used for the first trip and the tail
+  auto guarded_trip = [&](long long off) {
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) {
+        const long long p = off + s * STEP + lane * EPL + e;
+        if (p >= start && p < end) {
+          const unsigned ie = bidx[p];
+          const T pe = bval[p] * x[ie & col_mask];
+          lds_add(acc + (ie >> col_bits), pe);
+        }
+      }
+    }
+  };
+  long long off = first;
+  if (off < end) {
+    guarded_trip(off);
+    off += TRIP;
+  }
+  // interior trips: aligned vector loads, next trip prefetched
+  if (off + TRIP <= end) {
+    unsigned ci[STEPS][EPL];
+    T cv[STEPS][EPL];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) load_entries<NT>(bidx, bval, off + s * STEP + lane * EPL, ci[s], cv[s]);
+    for (; off + TRIP <= end; off += TRIP) {
+      unsigned ni[STEPS][EPL];
+      T nv[STEPS][EPL];
+      const bool more = off + 2 * TRIP <= end;
+      if (more) {
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s)
+          load_entries<NT>(bidx, bval, off + TRIP + s * STEP + lane * EPL, ni[s], nv[s]);
+      }
+      if (pace_fp) {
+        // time-triggered pacing: entry number k of a wavefront's range is not gathered
+        // before t0 + k * pace.  Wavefronts that run ahead wait here (the loads of the
+        // next trip are already in flight), so all of them cross x at the same pace and
+        // the part of x in use stays small enough for L2.  The clock only moves
+        // forward: the wait always ends.
+        const long long target = t0 + (((off - first) * (long long)pace_fp) >> 16);
+        while (wall_clock64() < target) __builtin_amdgcn_s_sleep(2);
+      }
+      T pr[STEPS][EPL];
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) pr[s][e] = cv[s][e] * x[ci[s][e] & col_mask];
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) lds_add(acc + (ci[s][e] >> col_bits), pr[s][e]);
+      if (more) {
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+          for (int e = 0; e < EPL; ++e) {
+            ci[s][e] = ni[s][e];
+            cv[s][e] = nv[s][e];
+          }
+      }
+    }
+  }
+  if (off < end) guarded_trip(off);
+  wave_lds_sync();
+  for (int i = lane; i < rows_here; i += 64) y[row0 + i] = acc[i] + y[row0 + i];
+}
+
+// key = (row block << (32 + slice bits)) | (slice << 32) | (row in block << col_bits) | column
+__global__ __launch_bounds__(256) void colblock_keys_kernel(int nrows, int col_bits, int slice_log2, int slice_bits,
+                                                            const int *__restrict__ pos,
+                                                            const int *__restrict__ crd,
+                                                            unsigned long long *__restrict__ keys) {
+  // one wavefront per row: coalesced over the row's entries
+  const int lane = threadIdx.x & 63;
+  const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= nrows) return;
+  const unsigned long long rb = (unsigned long long)(row / kColblockRows);
+  const unsigned long long rl = (unsigned long long)(row % kColblockRows);
+  const int s = pos[row], e = pos[row + 1];
+  for (int j = s + lane; j < e; j += 64) {
+    const unsigned long long c = (unsigned long long)(unsigned)crd[j];
+    keys[j] = (rb << (32 + slice_bits)) | ((c >> slice_log2) << 32) | (rl << col_bits) | c;
+  }
+}
+
+__global__ __launch_bounds__(256) void colblock_low_word_kernel(long long n, const unsigned long long *__restrict__ keys,
+                                                                unsigned *__restrict__ out) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) out[i] = (unsigned)keys[i];
+}
+
+void free_colblock(lapis_hip_csr_plan *p) {
+  if (p->colblock_idx) (void)hipFree(p->colblock_idx);
+  if (p->colblock_val) (void)hipFree(p->colblock_val);
+  p->colblock_idx = nullptr;
+  p->colblock_val = nullptr;
+  p->colblock_built = false;
+}
+
+template <typename T, int STEPS, int EPL, int PAD>
+int launch_colblock_cfg(const lapis_hip_csr_plan *p, const int *pos, const T *x, T *y, hipStream_t st) {
+  constexpr int WAVES = 4;
+  const int64_t nrb = ceil_div(p->stats.nrows, kColblockRows);
+  const dim3 grid((unsigned)ceil_div(nrb, WAVES)), block(64 * WAVES);
+  if (p->nontemporal)
+    launch_timed(spmv_colblock_kernel<T, kColblockRows, WAVES, STEPS, EPL, PAD, true>, grid, block, st,
+                 (int)p->stats.nrows, (int)p->stats.nnz, p->colblock_col_bits, pos,
+                 (const unsigned *)p->colblock_idx, (const T *)p->colblock_val, x, y, p->colblock_pace_fp);
+  else
+    launch_timed(spmv_colblock_kernel<T, kColblockRows, WAVES, STEPS, EPL, PAD, false>, grid, block, st,
+                 (int)p->stats.nrows, (int)p->stats.nnz, p->colblock_col_bits, pos,
+                 (const unsigned *)p->colblock_idx, (const T *)p->colblock_val, x, y, p->colblock_pace_fp);
+  LAPIS_LAUNCH_CHECK();
+  return LAPIS_HIP_OK;
+}
+
+template <typename T>
+int launch_colblock(const lapis_hip_csr_plan *p, const int *pos, const T *x, T *y, hipStream_t st) {
+  constexpr int PADW = (40960 - 4 * kColblockRows * (int)sizeof(T)) / (int)sizeof(T);  // 40 KB per workgroup
+  const int key = p->colblock_steps * 100 + p->colblock_epl * 10 + (p->colblock_pad ? 1 : 0);
+  switch (key) {
+    case 140: return launch_colblock_cfg<T, 1, 4, 0>(p, pos, x, y, st);
+    case 141: return launch_colblock_cfg<T, 1, 4, PADW>(p, pos, x, y, st);
+    case 240: return launch_colblock_cfg<T, 2, 4, 0>(p, pos, x, y, st);
+    case 241: return launch_colblock_cfg<T, 2, 4, PADW>(p, pos, x, y, st);
+    case 120: return launch_colblock_cfg<T, 1, 2, 0>(p, pos, x, y, st);
+    case 121: return launch_colblock_cfg<T, 1, 2, PADW>(p, pos, x, y, st);
+    case 220: return launch_colblock_cfg<T, 2, 2, 0>(p, pos, x, y, st);
+    case 221: return launch_colblock_cfg<T, 2, 2, PADW>(p, pos, x, y, st);
+    case 110: return launch_colblock_cfg<T, 1, 1, 0>(p, pos, x, y, st);
+    case 111: return launch_colblock_cfg<T, 1, 1, PADW>(p, pos, x, y, st);
+    case 210: return launch_colblock_cfg<T, 2, 1, 0>(p, pos, x, y, st);
+    case 211: return launch_colblock_cfg<T, 2, 1, PADW>(p, pos, x, y, st);
+    default:
+      return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT, "colblock: no kernel for steps=%d entries-per-lane=%d",
+                       p->colblock_steps, p->colblock_epl);
+  }
+}
+template int launch_colblock<double>(const lapis_hip_csr_plan *, const int *, const double *, double *, hipStream_t);
+template int launch_colblock<float>(const lapis_hip_csr_plan *, const int *, const float *, float *, hipStream_t);
+
+namespace {
+int bits_for(int64_t n) {  // bits needed for values 0..n-1
+  int b = 0;
+  while (b < 62 && (1LL << b) < n) ++b;
+  return b;
+}
+
+// Finds the pace (clock ticks per entry) at which the paced kernel runs fastest:
+// times the free-running kernel, then paced runs aimed at 50 % .. 95 % of that time,
+// and keeps the best (or no pacing if nothing beats the free run by 2 %).
+template <typename T>
+int calibrate_pace(lapis_hip_csr_plan *p, hipStream_t st) {
+  const int64_t nrows = p->stats.nrows, ncols = p->stats.ncols;
+  int dev = 0, clock_khz = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&clock_khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess || clock_khz <= 0)
+    return LAPIS_HIP_OK;  // no clock rate, no pacing
+  T *x = nullptr, *y = nullptr;
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  auto done = [&](int rc) {
+    if (x) (void)hipFree(x);
+    if (y) (void)hipFree(y);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    return rc;
+  };
+  if (hipMalloc(&x, sizeof(T) * (size_t)ncols) != hipSuccess || hipMalloc(&y, sizeof(T) * (size_t)nrows) != hipSuccess ||
+      hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)
+    return done(LAPIS_HIP_OK);
+  (void)hipMemsetAsync(x, 0, sizeof(T) * (size_t)ncols, st);
+  (void)hipMemsetAsync(y, 0, sizeof(T) * (size_t)nrows, st);
+  auto time_ms = [&](unsigned pace) -> double {
+    p->colblock_pace_fp = pace;
+    double best = 1e30;
+    for (int rep = 0; rep < 4; ++rep) {
+      (void)hipEventRecord(e0, st);
+      if (launch_colblock<T>(p, p->pos, x, y, st) != LAPIS_HIP_OK) return 1e30;
+      (void)hipEventRecord(e1, st);
+      if (hipEventSynchronize(e1) != hipSuccess) return 1e30;
+      float ms = 0.f;
+      (void)hipEventElapsedTime(&ms, e0, e1);
+      if (rep > 0) best = std::min<double>(best, ms);
+    }
+    return best;
+  };
+  const double free_ms = time_ms(0);
+  const double entries_per_wave = (double)p->stats.nnz / (double)ceil_div(nrows, kColblockRows);
+  unsigned best_pace = 0;
+  int best_pct = 0;
+  double best_ms = free_ms * 0.98;
+  auto try_pct = [&](int pct) {
+    const double target_ticks = free_ms * 1e-3 * (pct / 100.0) * (double)clock_khz * 1e3;
+    const double fp = target_ticks / entries_per_wave * 65536.0;
+    if (fp < 1.0 || fp > 4.0e9) return;
+    const double ms = time_ms((unsigned)fp);
+    if (getenv("LAPIS_HIP_VERBOSE")) fprintf(stderr, "lapis_hip:   pace target %d%% -> %.4f ms\n", pct, ms);
+    if (ms < best_ms) {
+      best_ms = ms;
+      best_pace = (unsigned)fp;
+      best_pct = pct;
+    }
+  };
+  for (int pct = 50; pct <= 95; pct += 5) try_pct(pct);  // coarse
+  if (best_pct) {
+    const int centre = best_pct;
+    for (int pct = centre - 4; pct <= centre + 4; ++pct)  // fine
+      if (pct != centre) try_pct(pct);
+  }
+  p->colblock_pace_fp = best_pace;
+  p->colblock_free_ms = free_ms;
+  p->colblock_paced_ms = best_pace ? best_ms : free_ms;
+  if (getenv("LAPIS_HIP_VERBOSE"))
+    fprintf(stderr, "lapis_hip: column-blocked SpMV calibration: free %.4f ms, paced %.4f ms at %.3f ticks/entry\n",
+            free_ms, p->colblock_paced_ms, best_pace / 65536.0);
+  return done(LAPIS_HIP_OK);
+}
+
+template <typename T>
+int build(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int slice_log2, hipStream_t st) {
+  const int64_t nnz = p->stats.nnz, nrows = p->stats.nrows;
+  const int col_bits = std::max(1, bits_for(p->stats.ncols));
+  const int rb_bits = bits_for(ceil_div(nrows, kColblockRows));
+  // the 64-bit sort key holds row block | slice | 32-bit entry word: slices must be
+  // coarse enough for all three to fit
+  slice_log2 = std::max(slice_log2, col_bits - (32 - rb_bits));
+  const int slice_bits = std::max(0, col_bits - slice_log2);
+  const int end_bit = 32 + slice_bits + rb_bits;
+  if (end_bit > 64 || slice_log2 < 0 || slice_log2 > 31)
+    return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT, "csr_plan_build_colblock: sort key needs %d bits", end_bit);
+
+  unsigned long long *keys_in = nullptr, *keys_out = nullptr;
+  T *val_out = nullptr;
+  unsigned *idx = nullptr;
+  void *temp = nullptr;
+  size_t temp_bytes = 0;
+  auto fail = [&](hipError_t e, const char *what) {
+    if (keys_in) (void)hipFree(keys_in);
+    if (keys_out) (void)hipFree(keys_out);
+    if (val_out) (void)hipFree(val_out);
+    if (idx) (void)hipFree(idx);
+    if (temp) (void)hipFree(temp);
+    return set_error(LAPIS_HIP_ERR_RUNTIME, "csr_plan_build_colblock: %s failed: %s", what, hipGetErrorString(e));
+  };
+  hipError_t e;
+  if ((e = hipMalloc(&keys_in, sizeof(unsigned long long) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
+  if ((e = hipMalloc(&keys_out, sizeof(unsigned long long) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
+  if ((e = hipMalloc(&val_out, sizeof(T) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
+  if ((e = hipMalloc(&idx, sizeof(unsigned) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
+  hipLaunchKernelGGL(colblock_keys_kernel, dim3((unsigned)ceil_div(nrows, 4)), dim3(256), 0, st, (int)nrows, col_bits,
+                     slice_log2, slice_bits, p->pos, crd, keys_in);
+  if ((e = hipGetLastError()) != hipSuccess) return fail(e, "key kernel");
+  if ((e = hipcub::DeviceRadixSort::SortPairs(nullptr, temp_bytes, keys_in, keys_out, val, val_out, (int)nnz, 0,
+                                              end_bit, st)) != hipSuccess)
+    return fail(e, "radix sort sizing");
+  if ((e = hipMalloc(&temp, temp_bytes ? temp_bytes : 1)) != hipSuccess) return fail(e, "hipMalloc");
+  if ((e = hipcub::DeviceRadixSort::SortPairs(temp, temp_bytes, keys_in, keys_out, val, val_out, (int)nnz, 0, end_bit,
+                                              st)) != hipSuccess)
+    return fail(e, "radix sort");
+  hipLaunchKernelGGL(colblock_low_word_kernel, dim3((unsigned)ceil_div(nnz, 256)), dim3(256), 0, st, (long long)nnz,
+                     keys_out, idx);
+  if ((e = hipGetLastError()) != hipSuccess) return fail(e, "index kernel");
+  if ((e = hipStreamSynchronize(st)) != hipSuccess) return fail(e, "synchronize");
+  (void)hipFree(keys_in);
+  (void)hipFree(keys_out);
+  (void)hipFree(temp);
+  free_colblock(p);
+  {
+    const char *stp = getenv("LAPIS_HIP_COLBLOCK_STEPS"), *epl = getenv("LAPIS_HIP_COLBLOCK_EPL"),
+               *pad = getenv("LAPIS_HIP_COLBLOCK_PAD");
+    p->colblock_steps = stp ? atoi(stp) : 2;
+    p->colblock_epl = epl ? atoi(epl) : 2;
+    p->colblock_pad = pad ? atoi(pad) : 0;
+  }
+  p->colblock_idx = idx;
+  p->colblock_val = val_out;
+  p->colblock_value_bytes = (int)sizeof(T);
+  p->colblock_col_bits = col_bits;
+  p->colblock_slice_log2 = slice_log2;
+  p->colblock_built = true;
+  p->colblock_pace_fp = 0;
+  const char *pace_env = getenv("LAPIS_HIP_COLBLOCK_PACE");
+  if (pace_env && atoi(pace_env) == 0) return LAPIS_HIP_OK;
+  return calibrate_pace<T>(p, st);
+}
+}  // namespace
+
+}  // namespace lapis
+
+using namespace lapis;
+
+extern "C" int lapis_hip_csr_plan_build_colblock(lapis_hip_csr_plan *plan, const int32_t *crd, const void *val,
+                                                 int value_bytes, int slice_log2_cols, lapis_hip_stream_t stream) {
+  LAPIS_CHECK_INIT();
+  LAPIS_REQUIRE(plan, "csr_plan_build_colblock: null plan");
+  LAPIS_REQUIRE(value_bytes == 4 || value_bytes == 8, "csr_plan_build_colblock: value_bytes must be 4 or 8");
+  const lapis_hip_csr_stats &s = plan->stats;
+  LAPIS_REQUIRE(s.nnz > 0, "csr_plan_build_colblock: the matrix has no non-zeros");
+  LAPIS_REQUIRE(crd && val, "csr_plan_build_colblock: null coordinates or values");
+  int col_bits = 1;
+  while ((1LL << col_bits) < s.ncols) ++col_bits;
+  if (col_bits + kColblockRowBits > 32)
+    return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT,
+                     "csr_plan_build_colblock: %lld columns need %d bits, more than the %d an entry has room for",
+                     (long long)s.ncols, col_bits, 32 - kColblockRowBits);
+  if (slice_log2_cols <= 0) slice_log2_cols = value_bytes == 8 ? 17 : 18;  // 1 MB of x per slice
+  slice_log2_cols = std::min(slice_log2_cols, col_bits);
+  hipStream_t st = as_stream(stream);
+  const int rc = value_bytes == 8 ? build<double>(plan, crd, static_cast<const double *>(val), slice_log2_cols, st)
+                                  : build<float>(plan, crd, static_cast<const float *>(val), slice_log2_cols, st);
+  if (rc == LAPIS_HIP_OK) {
+    plan->stats.kernel = LAPIS_HIP_SPMV_COLBLOCK;
+    plan->stats.width = 0;
+    plan->stats.chunk = 0;
+  }
+  return rc;
+}

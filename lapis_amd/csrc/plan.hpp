@@ -1,0 +1,41 @@
+// The CSR plan object behind lapis_hip_csr_plan (opaque in the C ABI).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "lapis_hip.h"
+
+struct lapis_hip_csr_plan {
+  lapis_hip_csr_stats stats;
+  const int32_t *pos;
+  int nchunks;
+  bool nontemporal;
+  // row-split (NNZSPLIT) metadata
+  int *chunk_row;    // device, int[nchunks+1]
+  void *part_first;  // device, 8 bytes * nchunks
+  void *part_last;   // device, 8 bytes * nchunks
+  // column-blocked (COLBLOCK) copy of the matrix, built on request
+  bool colblock_built;
+  int colblock_value_bytes;
+  int colblock_col_bits;     // low bits of an entry hold the column, the bits above the row inside its row block
+  int colblock_slice_log2;   // columns per x slice = 1 << this
+  unsigned *colblock_idx;    // device, uint32[nnz]
+  void *colblock_val;        // device, T[nnz]
+  int colblock_steps;        // steps per wavefront trip
+  int colblock_epl;          // entries per lane per step (1, 2 or 4)
+  int colblock_pad;          // pad LDS so that exactly four workgroups fit a CU
+  unsigned colblock_pace_fp; // clock ticks per entry (16.16 fixed point) of the time-triggered pacing, 0 = off
+  double colblock_free_ms;   // calibration: kernel time without pacing
+  double colblock_paced_ms;  // calibration: kernel time at the chosen pace
+};
+
+namespace lapis {
+constexpr int kColblockRows = 1024;  // rows per wavefront in the column-blocked kernel
+constexpr int kColblockRowBits = 10;
+
+// Launches the column-blocked kernel; defined in colblock.hip.
+template <typename T>
+int launch_colblock(const lapis_hip_csr_plan *plan, const int *pos, const T *x, T *y, hipStream_t st);
+void free_colblock(lapis_hip_csr_plan *plan);
+}  // namespace lapis

@@ -11,6 +11,7 @@
 #include <cstring>
 
 #include "common.hpp"
+#include "plan.hpp"
 
 namespace lapis {
 
@@ -296,6 +297,7 @@ struct DeviceStats {
   int pad;
   unsigned long long empty_rows;
   double sum_sq;
+  unsigned long long span_sum;  // sum over 1024-non-zero chunks of (max column - min column)
 };
 
 __global__ __launch_bounds__(256) void row_stats_kernel(int nrows, const int *__restrict__ pos,
@@ -329,15 +331,32 @@ __global__ __launch_bounds__(256) void row_stats_kernel(int nrows, const int *__
   }
 }
 
+// One wavefront per 1024 consecutive non-zeros: range check of the coordinates and
+// the column span (max - min) of the chunk, summed over chunks.  The mean span says
+// how much of x a wavefront's gathers wander over: small for stencils and bands,
+// the whole vector for uniformly random columns.
 __global__ __launch_bounds__(256) void crd_range_kernel(long long nnz, int ncols,
                                                         const int *__restrict__ crd, DeviceStats *st) {
-  int bad = 0;
-  for (long long j = (long long)blockIdx.x * 256 + threadIdx.x; j < nnz;
-       j += (long long)gridDim.x * 256) {
-    const int cj = crd[j];
+  const int lane = threadIdx.x & 63;
+  const long long chunk = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const long long j0 = chunk * 1024;
+  if (j0 >= nnz) return;
+  int mn = INT32_MAX, mx = INT32_MIN, bad = 0;
+  for (int k = lane; k < 1024 && j0 + k < nnz; k += 64) {
+    const int cj = crd[j0 + k];
     if (cj < 0 || cj >= ncols) bad = 1;
+    mn = std::min(mn, cj);
+    mx = std::max(mx, cj);
   }
-  if (__ballot(bad) && (threadIdx.x & 63) == 0) atomicOr(&st->bad, 2);
+  for (int o = 32; o > 0; o >>= 1) {
+    mn = std::min(mn, __shfl_xor(mn, o, 64));
+    mx = std::max(mx, __shfl_xor(mx, o, 64));
+    bad |= __shfl_xor(bad, o, 64);
+  }
+  if (lane == 0) {
+    if (bad) atomicOr(&st->bad, 2);
+    atomicAdd(&st->span_sum, (unsigned long long)((long long)mx - (long long)mn));
+  }
 }
 
 template <int CH>
@@ -387,16 +406,6 @@ int64_t reference_hint(int64_t nrows, int64_t pos_first, int64_t pos_last) {
   return (pos_last - pos_first + nrows - 1) / nrows;
 }
 }  // namespace
-
-struct lapis_hip_csr_plan {
-  lapis_hip_csr_stats stats;
-  const int32_t *pos;
-  int nchunks;
-  bool nontemporal;
-  int *chunk_row;     // device, int[nchunks+1]
-  void *part_first;   // device, 8 bytes * nchunks
-  void *part_last;    // device, 8 bytes * nchunks
-};
 
 namespace {
 
@@ -532,6 +541,11 @@ int spmv_impl(lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, const int3
         return nt ? launch_nnzsplit<T, true, true>(plan, pos, crd, val, x, y, st)
                   : launch_nnzsplit<T, true, false>(plan, pos, crd, val, x, y, st);
       return launch_nnzsplit<T, false, true>(plan, pos, crd, val, x, y, st);
+    case LAPIS_HIP_SPMV_COLBLOCK:
+      if (!plan->colblock_built || plan->colblock_value_bytes != (int)sizeof(T))
+        return set_error(LAPIS_HIP_ERR_PLAN_MISMATCH, "spmv: the plan holds no column-blocked copy for %d-byte values",
+                         (int)sizeof(T));
+      return launch_colblock<T>(plan, pos, x, y, st);
     default:
       return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT, "spmv: plan holds unknown kernel %d", s.kernel);
   }
@@ -543,6 +557,7 @@ void free_plan_buffers(lapis_hip_csr_plan *p) {
   if (p->part_last) (void)hipFree(p->part_last);
   p->chunk_row = nullptr;
   p->part_first = p->part_last = nullptr;
+  free_colblock(p);
 }
 
 }  // namespace
@@ -568,7 +583,7 @@ extern "C" int lapis_hip_csr_plan_create(lapis_hip_csr_plan **out, int64_t nrows
     return set_error(LAPIS_HIP_ERR_BAD_CSR, "csr_plan_create: pos[0]=%d pos[n]=%d, expected 0 and nnz=%lld",
                      ends[0], ends[1], (long long)nnz);
 
-  DeviceStats init{INT32_MAX, 0, 0, 0, 0ull, 0.0};
+  DeviceStats init{INT32_MAX, 0, 0, 0, 0ull, 0.0, 0ull};
   DeviceStats host = init;
   if (nrows > 0) {
     DeviceStats *dstats = nullptr;
@@ -580,7 +595,7 @@ extern "C" int lapis_hip_csr_plan_create(lapis_hip_csr_plan **out, int64_t nrows
       e = hipGetLastError();
     }
     if (e == hipSuccess && crd && nnz > 0) {
-      const int blocks = (int)std::min<int64_t>(ceil_div(nnz, 256), 8192);
+      const int blocks = (int)ceil_div(ceil_div(nnz, 1024), 4);
       hipLaunchKernelGGL(crd_range_kernel, dim3(blocks), dim3(256), 0, st, (long long)nnz, (int)ncols, crd,
                          dstats);
       e = hipGetLastError();
@@ -608,6 +623,18 @@ extern "C" int lapis_hip_csr_plan_create(lapis_hip_csr_plan **out, int64_t nrows
   s.empty_rows = (int64_t)host.empty_rows;
   s.mean_row_len = nrows ? (double)nnz / (double)nrows : 0.0;
   s.var_row_len = nrows ? std::max(0.0, host.sum_sq / (double)nrows - s.mean_row_len * s.mean_row_len) : 0.0;
+  s.mean_chunk_col_span = (crd && nnz > 0) ? (double)host.span_sum / (double)ceil_div(nnz, 1024) : -1.0;
+  // The column-blocked copy pays when the gathers of a chunk wander over more of x
+  // than an XCD's L2 keeps (4 MB, shared with the streamed arrays), the rows are even
+  // enough for equal row blocks to mean equal work, and the entry encoding fits.
+  {
+    int col_bits = 1;
+    while ((1LL << col_bits) < ncols) ++col_bits;
+    s.colblock_recommended = (s.mean_chunk_col_span * value_bytes > 2.0 * 1024 * 1024 && col_bits <= 22 &&
+                              nnz >= (1 << 20) && (double)s.max_row_len <= 64.0 * std::max(1.0, s.mean_row_len))
+                                 ? 1
+                                 : 0;
+  }
   s.reference_hint = reference_hint(nrows, ends[0], ends[1]);
   s.reference_vector_length = reference_vector_length(s.reference_hint);
   p->pos = pos;
@@ -662,6 +689,14 @@ extern "C" int lapis_hip_csr_plan_set_kernel(lapis_hip_csr_plan *plan, int kerne
       s.kernel = kernel;
       s.width = 0;
       s.chunk = kChunk;
+      return LAPIS_HIP_OK;
+    case LAPIS_HIP_SPMV_COLBLOCK:
+      if (!plan->colblock_built)
+        return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT,
+                         "csr_plan_set_kernel: call lapis_hip_csr_plan_build_colblock first");
+      s.kernel = kernel;
+      s.width = 0;
+      s.chunk = 0;
       return LAPIS_HIP_OK;
     default:
       return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT, "csr_plan_set_kernel: unknown kernel %d", kernel);

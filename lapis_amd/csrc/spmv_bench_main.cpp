@@ -1,0 +1,208 @@
+// SpMV benchmark driver over a MatrixMarket file, the counterpart of the
+// reference's benchmarks/spmv/main.cpp: read the matrix, keep it resident on the
+// device, one warm-up call, then `trials` calls each followed by a fence, print the
+// mean time.  Usage: lapis_spmv_bench matrix.mtx [trials=1000] [kernel]
+//   kernel: auto (default) | reference | subwarpN | rowblock | nnzsplit | colblock
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <chrono>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <iostream>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include "lapis_hip.h"
+
+namespace {
+
+struct Csr {
+  int64_t nrows = 0, ncols = 0;
+  std::vector<int32_t> pos, crd;
+  std::vector<double> val;
+};
+
+bool read_matrix_market(const std::string &path, Csr &A, std::string &err) {
+  std::ifstream in(path);
+  if (!in) {
+    err = "cannot open " + path;
+    return false;
+  }
+  std::string line;
+  if (!std::getline(in, line) || line.rfind("%%MatrixMarket", 0) != 0) {
+    err = "not a MatrixMarket file";
+    return false;
+  }
+  std::string banner, object, format, field, symmetry;
+  {
+    std::istringstream hs(line);
+    hs >> banner >> object >> format >> field >> symmetry;
+  }
+  auto lower = [](std::string s) {
+    std::transform(s.begin(), s.end(), s.begin(), ::tolower);
+    return s;
+  };
+  format = lower(format);
+  field = lower(field);
+  symmetry = lower(symmetry);
+  if (lower(object) != "matrix" || format != "coordinate") {
+    err = "only 'matrix coordinate' files are supported";
+    return false;
+  }
+  if (field != "real" && field != "integer" && field != "pattern" && field != "double") {
+    err = "unsupported field type " + field;
+    return false;
+  }
+  const bool pattern = field == "pattern";
+  const bool sym = symmetry == "symmetric", skew = symmetry == "skew-symmetric";
+  if (!sym && !skew && symmetry != "general") {
+    err = "unsupported symmetry " + symmetry;
+    return false;
+  }
+  while (std::getline(in, line))
+    if (!line.empty() && line[0] != '%') break;
+  long long m = 0, n = 0, entries = 0;
+  if (sscanf(line.c_str(), "%lld %lld %lld", &m, &n, &entries) != 3 || m < 0 || n < 0 || entries < 0) {
+    err = "bad size line";
+    return false;
+  }
+  struct Entry {
+    int32_t r, c;
+    double v;
+  };
+  std::vector<Entry> coo;
+  coo.reserve((size_t)entries * ((sym || skew) ? 2 : 1));
+  for (long long k = 0; k < entries; ++k) {
+    long long r, c;
+    double v = 1.0;
+    if (!(in >> r >> c)) {
+      err = "file ends before all entries were read";
+      return false;
+    }
+    if (!pattern && !(in >> v)) {
+      err = "missing value";
+      return false;
+    }
+    if (r < 1 || r > m || c < 1 || c > n) {
+      err = "entry outside the matrix";
+      return false;
+    }
+    coo.push_back({(int32_t)(r - 1), (int32_t)(c - 1), v});
+    if ((sym || skew) && r != c) coo.push_back({(int32_t)(c - 1), (int32_t)(r - 1), skew ? -v : v});
+  }
+  if (coo.size() > (size_t)INT32_MAX) {
+    err = "more non-zeros than int32 positions can address";
+    return false;
+  }
+  std::sort(coo.begin(), coo.end(), [](const Entry &a, const Entry &b) { return a.r != b.r ? a.r < b.r : a.c < b.c; });
+  A.nrows = m;
+  A.ncols = n;
+  A.pos.assign((size_t)m + 1, 0);
+  A.crd.resize(coo.size());
+  A.val.resize(coo.size());
+  for (size_t k = 0; k < coo.size(); ++k) {
+    A.pos[(size_t)coo[k].r + 1]++;
+    A.crd[k] = coo[k].c;
+    A.val[k] = coo[k].v;
+  }
+  for (int64_t i = 0; i < m; ++i) A.pos[(size_t)i + 1] += A.pos[(size_t)i];
+  return true;
+}
+
+#define CHECK_HIP(expr)                                                              \
+  do {                                                                               \
+    hipError_t e_ = (expr);                                                          \
+    if (e_ != hipSuccess) {                                                          \
+      fprintf(stderr, "%s failed: %s\n", #expr, hipGetErrorString(e_));              \
+      return 2;                                                                      \
+    }                                                                                \
+  } while (0)
+#define CHECK_LAPIS(expr)                                                            \
+  do {                                                                               \
+    int s_ = (expr);                                                                 \
+    if (s_ != LAPIS_HIP_OK) {                                                        \
+      fprintf(stderr, "%s failed: %s: %s\n", #expr, lapis_hip_status_name(s_), lapis_hip_last_error()); \
+      return 2;                                                                      \
+    }                                                                                \
+  } while (0)
+
+}  // namespace
+
+int main(int argc, const char **argv) {
+  if (argc < 2 || argc > 4) {
+    std::cout << "Expected: matrix file in MatrixMarket format [trials] [kernel]\n";
+    return 1;
+  }
+  const std::string mfile = argv[1];
+  const int trials = argc > 2 ? std::max(1, atoi(argv[2])) : 1000;
+  const std::string kernel = argc > 3 ? argv[3] : "auto";
+  CHECK_LAPIS(lapis_hip_init());
+  std::cout << "Reading matrix from " << mfile << "...\n";
+  Csr A;
+  std::string err;
+  if (!read_matrix_market(mfile, A, err)) {
+    std::cerr << "error: " << err << "\n";
+    return 1;
+  }
+  const int64_t nnz = (int64_t)A.crd.size();
+  std::cout << "Read matrix (" << A.nrows << "x" << A.ncols << " with " << nnz << " entries)\n";
+
+  int32_t *pos = nullptr, *crd = nullptr;
+  double *val = nullptr, *x = nullptr, *y = nullptr;
+  CHECK_HIP(hipMalloc(&pos, sizeof(int32_t) * (A.nrows + 1)));
+  CHECK_HIP(hipMalloc(&crd, sizeof(int32_t) * std::max<int64_t>(nnz, 1)));
+  CHECK_HIP(hipMalloc(&val, sizeof(double) * std::max<int64_t>(nnz, 1)));
+  CHECK_HIP(hipMalloc(&x, sizeof(double) * std::max<int64_t>(A.ncols, 1)));
+  CHECK_HIP(hipMalloc(&y, sizeof(double) * std::max<int64_t>(A.nrows, 1)));
+  CHECK_HIP(hipMemcpy(pos, A.pos.data(), sizeof(int32_t) * (A.nrows + 1), hipMemcpyHostToDevice));
+  CHECK_HIP(hipMemcpy(crd, A.crd.data(), sizeof(int32_t) * nnz, hipMemcpyHostToDevice));
+  CHECK_HIP(hipMemcpy(val, A.val.data(), sizeof(double) * nnz, hipMemcpyHostToDevice));
+  // x and y start at zero, as the Kokkos views of the reference driver do
+  CHECK_HIP(hipMemset(x, 0, sizeof(double) * std::max<int64_t>(A.ncols, 1)));
+  CHECK_HIP(hipMemset(y, 0, sizeof(double) * std::max<int64_t>(A.nrows, 1)));
+
+  lapis_hip_csr_plan *plan = nullptr;
+  if (kernel != "reference") {
+    CHECK_LAPIS(lapis_hip_csr_plan_create(&plan, A.nrows, A.ncols, nnz, pos, crd, 8, nullptr));
+    if (kernel == "rowblock") CHECK_LAPIS(lapis_hip_csr_plan_set_kernel(plan, LAPIS_HIP_SPMV_ROWBLOCK, 0));
+    else if (kernel == "nnzsplit") CHECK_LAPIS(lapis_hip_csr_plan_set_kernel(plan, LAPIS_HIP_SPMV_NNZSPLIT, 0));
+    else if (kernel == "colblock") CHECK_LAPIS(lapis_hip_csr_plan_build_colblock(plan, crd, val, 8, 0, nullptr));
+    else if (kernel.rfind("subwarp", 0) == 0)
+      CHECK_LAPIS(lapis_hip_csr_plan_set_kernel(plan, LAPIS_HIP_SPMV_SUBWARP, atoi(kernel.c_str() + 7)));
+    else if (kernel != "auto") {
+      std::cerr << "unknown kernel " << kernel << "\n";
+      return 1;
+    }
+    lapis_hip_csr_stats s;
+    CHECK_LAPIS(lapis_hip_csr_plan_get_stats(plan, &s));
+    std::cout << "rows: min " << s.min_row_len << " mean " << s.mean_row_len << " max " << s.max_row_len
+              << "; kernel " << s.kernel << " width " << s.width << "; reference vector length "
+              << s.reference_vector_length << "\n";
+  }
+  // Warmup
+  CHECK_LAPIS(lapis_hip_spmv_csr_f64_i32(plan, A.nrows, A.ncols, pos, crd, val, x, y, nullptr));
+  CHECK_LAPIS(lapis_hip_stream_synchronize(nullptr));
+  const auto t0 = std::chrono::steady_clock::now();
+  for (int i = 0; i < trials; i++) {
+    CHECK_LAPIS(lapis_hip_spmv_csr_f64_i32(plan, A.nrows, A.ncols, pos, crd, val, x, y, nullptr));
+    CHECK_LAPIS(lapis_hip_stream_synchronize(nullptr));
+  }
+  const double elapsed = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+  const double avg = elapsed / trials;
+  const double bytes = 2.0 * 8 * A.nrows + 12.0 * nnz + 4.0 * (A.nrows + 1);  // benchmarks/plots/plotSPMV.py:20
+  std::cout << "spmv avg time = " << avg << "\n";
+  std::cout << "bandwidth = " << bytes / avg / 1e9 << " GB/s, " << 2.0 * nnz / avg / 1e9 << " GFLOP/s\n";
+  lapis_hip_csr_plan_destroy(plan);
+  (void)hipFree(pos);
+  (void)hipFree(crd);
+  (void)hipFree(val);
+  (void)hipFree(x);
+  (void)hipFree(y);
+  lapis_hip_finalize();
+  return 0;
+}

@@ -98,6 +98,38 @@ def laplace3d(nx, dtype=np.float64):
     return CSR(n, n, _pos_from_lengths(ok.sum(axis=1, dtype=np.int64)), crd, np.ascontiguousarray(val))
 
 
+def elasticity3d(nx, dtype=np.float64):
+    """Structure of a 3-D elasticity operator on an nx^3 node grid: 3 unknowns per node,
+    27-point node stencil, a full 3x3 block per node pair (rows 3*nx^3, nnz 9*(3nx-2)^3).
+    nx = 60 gives the size of the reference's published matrix Elasticity3D_60
+    (648 000 rows, 50 757 768 non-zeros, benchmarks/plots/plotSPMV.py:14-15); the values
+    (diagonal 100, rest -1) are stand-ins, SpMV time does not depend on them."""
+    n = nx ** 3
+    idx = np.arange(n, dtype=np.int64)
+    ix, iy, iz = idx % nx, (idx // nx) % nx, idx // (nx * nx)
+    cands, oks = [], []
+    for dz in (-1, 0, 1):
+        for dy in (-1, 0, 1):
+            for dx in (-1, 0, 1):
+                ok = ((ix + dx >= 0) & (ix + dx < nx) & (iy + dy >= 0) & (iy + dy < nx) & (iz + dz >= 0) & (iz + dz < nx))
+                cands.append(idx + dx + dy * nx + dz * nx * nx)
+                oks.append(ok)
+    cand = np.stack(cands, axis=1)
+    ok = np.stack(oks, axis=1)
+    nb = cand[ok]                                   # neighbour nodes, node-major, ascending inside a node
+    cnt = ok.sum(axis=1)                            # neighbours per node
+    node_start = np.zeros(n + 1, dtype=np.int64)
+    np.cumsum(cnt, out=node_start[1:])
+    row_len = np.repeat(3 * cnt, 3)                 # three rows per node, 3 columns per neighbour
+    pos = _pos_from_lengths(row_len)
+    nnz = int(pos[-1])
+    row_of = np.repeat(np.arange(3 * n, dtype=np.int64), row_len)
+    k = np.arange(nnz, dtype=np.int64) - pos[:-1].astype(np.int64)[row_of]
+    crd = (nb[node_start[row_of // 3] + k // 3] * 3 + k % 3).astype(np.int32)
+    val = np.where(crd == row_of, 100.0, -1.0).astype(dtype)
+    return CSR(3 * n, 3 * n, pos, crd, val)
+
+
 def poisson_random(n, mean=16.0, seed=2002, dtype=np.float64):
     """Square matrix, row length ~ Poisson(mean), uniform distinct sorted columns, values U[-1,1)."""
     rng = _rng(seed)
@@ -178,6 +210,14 @@ def config4(scale=1.0, k=64):
     n = max(64, int(1048576 * scale))
     A = fixed_degree_random(n, 32, seed=4004)
     return A, uniform_matrix(n, k, 4004 + 1)
+
+
+# Matrices of the reference's published SpMV table whose structure is a formula
+# (benchmarks/plots/spmv.csv:3,8): name -> (maker, published mean seconds on MI300A, on H100)
+PUBLISHED = {
+    "Laplace3D_100": (lambda: laplace3d(100), 5.44e-05, 7.29e-05),
+    "Elasticity3D_60": (lambda: elasticity3d(60), 2.85281e-04, 2.65587e-04),
+}
 
 
 def config5(scale=1.0):

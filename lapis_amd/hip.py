@@ -11,8 +11,9 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "liblapis_hip.so")
 
-SPMV_AUTO, SPMV_SUBWARP, SPMV_ROWBLOCK, SPMV_NNZSPLIT = 0, 1, 2, 3
-KERNEL_NAMES = {SPMV_AUTO: "auto", SPMV_SUBWARP: "subwarp", SPMV_ROWBLOCK: "rowblock", SPMV_NNZSPLIT: "nnzsplit"}
+SPMV_AUTO, SPMV_SUBWARP, SPMV_ROWBLOCK, SPMV_NNZSPLIT, SPMV_COLBLOCK = 0, 1, 2, 3, 4
+KERNEL_NAMES = {SPMV_AUTO: "auto", SPMV_SUBWARP: "subwarp", SPMV_ROWBLOCK: "rowblock", SPMV_NNZSPLIT: "nnzsplit",
+                SPMV_COLBLOCK: "colblock"}
 
 _i64, _u64, _vp, _int = ctypes.c_int64, ctypes.c_uint64, ctypes.c_void_p, ctypes.c_int
 _dbl, _flt = ctypes.c_double, ctypes.c_float
@@ -28,9 +29,10 @@ class LapisHipError(RuntimeError):
 class CsrStats(ctypes.Structure):
     _fields_ = [("nrows", _i64), ("ncols", _i64), ("nnz", _i64),
                 ("min_row_len", _i64), ("max_row_len", _i64), ("empty_rows", _i64),
-                ("mean_row_len", _dbl), ("var_row_len", _dbl),
+                ("mean_row_len", _dbl), ("var_row_len", _dbl), ("mean_chunk_col_span", _dbl),
                 ("reference_hint", _i64), ("reference_vector_length", ctypes.c_int32),
-                ("kernel", ctypes.c_int32), ("width", ctypes.c_int32), ("chunk", ctypes.c_int32)]
+                ("kernel", ctypes.c_int32), ("width", ctypes.c_int32), ("chunk", ctypes.c_int32),
+                ("colblock_recommended", ctypes.c_int32), ("reserved", ctypes.c_int32)]
 
     def as_dict(self):
         d = {k: getattr(self, k) for k, _ in self._fields_}
@@ -49,6 +51,7 @@ _SIGNATURES = {
     "lapis_hip_csr_plan_set_kernel": [_vp, _int, _int],
     "lapis_hip_csr_plan_get_stats": [_vp, ctypes.POINTER(CsrStats)],
     "lapis_hip_csr_plan_destroy": [_vp],
+    "lapis_hip_csr_plan_build_colblock": [_vp, _vp, _vp, _int, _int, _vp],
     "lapis_hip_spmv_csr_f64_i32": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp],
     "lapis_hip_spmv_csr_f32_i32": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp],
     "lapis_hip_spmm_csr_f32_i32": [_i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp],
@@ -167,6 +170,12 @@ class CsrPlan:
     def set_kernel(self, kernel, width=0):
         check(self._lib.lapis_hip_csr_plan_set_kernel(self._handle, kernel, width))
         return self
+
+    def build_colblock(self, crd, val, slice_log2_cols=0, stream=None):
+        """Copy the matrix into the column-blocked layout and select that kernel."""
+        check(self._lib.lapis_hip_csr_plan_build_colblock(self._handle, _ptr(crd), _ptr(val), val.element_size(),
+                                                          slice_log2_cols, _stream(stream)))
+        return self.set_kernel(SPMV_COLBLOCK)
 
     def destroy(self):
         if self._handle:

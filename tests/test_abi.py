@@ -52,8 +52,8 @@ def test_status_names_are_distinct():
 
 
 def test_stats_struct_matches_header_layout():
-    # 6 int64 + 2 double + int64 + 4 int32 = 88 bytes, no padding surprises
-    assert ctypes.sizeof(hip.CsrStats) == 6 * 8 + 2 * 8 + 8 + 4 * 4
+    # 6 int64 + 3 double + int64 + 6 int32 = 104 bytes, no padding surprises
+    assert ctypes.sizeof(hip.CsrStats) == 6 * 8 + 3 * 8 + 8 + 6 * 4
 
 
 @pytest.mark.parametrize("dtype", [np.float64, np.float32, np.int32])

@@ -24,9 +24,15 @@ def _spmv_full(gpu, oracle, A, x, dtype):
     plan = gpu.CsrPlan(A.nrows, A.ncols, pos, crd, value_bytes=np.dtype(dtype).itemsize)
     tdt = torch.float64 if dtype == np.float64 else torch.float32
     results = {}
-    for kid, width, name in ((0, 0, "auto"), (1, 0, "reference-width"), (2, 0, "rowblock"), (3, 0, "nnzsplit")):
+    variants = [(0, 0, "auto"), (1, 0, "reference-width"), (2, 0, "rowblock"), (3, 0, "nnzsplit")]
+    if A.ncols <= (1 << 22):
+        variants.append((4, 0, "colblock"))
+    for kid, width, name in variants:
         print("full-size", name, flush=True)
-        plan.set_kernel(kid, width)
+        if kid == 4:
+            plan.build_colblock(crd, val)
+        else:
+            plan.set_kernel(kid, width)
         y = torch.zeros(A.nrows, dtype=tdt, device="cuda")
         gpu.spmv(plan, A.nrows, A.ncols, pos, crd, val, dx, y)
         torch.cuda.synchronize()
