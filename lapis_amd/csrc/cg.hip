@@ -13,6 +13,7 @@
 
 #include "blas1.hpp"
 #include "common.hpp"
+#include "plan.hpp"
 
 namespace lapis {
 
@@ -168,9 +169,9 @@ __global__ __launch_bounds__(256) void cg_precond_kernel(long long n, const doub
   }
 }
 
-// p = z + beta p with beta = rz_next/rz; block 0 then rolls the scalars forward.
-// Every block reads rz and rz_next before any block can have rolled them: the roll
-// happens in a separate one-thread kernel queued behind this one.
+// p = z + beta p with beta = rz_next/rz.  The scalars are rolled forward
+// (rz = rz_next, i = i+1) by a separate one-thread kernel queued behind this one, so
+// that every block of this kernel still reads the pair it needs.
 __global__ __launch_bounds__(256) void cg_update_p_kernel(long long n, const double *__restrict__ z,
                                                           double *__restrict__ p, const CgState *st) {
   if (st->done) return;
@@ -282,8 +283,8 @@ extern "C" int lapis_hip_pcg_f64_i32(lapis_hip_csr_plan *plan, int64_t n, const 
                        (unsigned long long)launched);
     }
     for (int it = 0; it < todo; ++it) {
-      PCG_RC(lapis_hip_fill_f64(n, 0.0, Ap, stream));
-      PCG_RC(lapis_hip_spmv_csr_f64_i32(plan, n, n, pos, crd, val, p, Ap, stream));
+      // Ap = A p: the reference zero-fills Ap and accumulates (examples/pcg_solve.py:12-19)
+      PCG_RC(spmv_overwrite_f64(plan, n, n, pos, crd, val, p, Ap, stream));
       hipLaunchKernelGGL(cg_pap_kernel, dim3(grid), dim3(256), 0, st, (long long)n, p, Ap, state, partials);
       hipLaunchKernelGGL(cg_update_xr_kernel, dim3(grid), dim3(256), 0, st, (long long)n, p, Ap, x, r, state,
                          partials, pre);

@@ -38,4 +38,9 @@ constexpr int kColblockRowBits = 10;
 template <typename T>
 int launch_colblock(const lapis_hip_csr_plan *plan, const int *pos, const T *x, T *y, hipStream_t st);
 void free_colblock(lapis_hip_csr_plan *plan);
+
+// y = A x without reading y; defined in spmv.hip.
+int spmv_overwrite_f64(lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, const int32_t *pos,
+                       const int32_t *crd, const double *val, const double *x, double *y,
+                       lapis_hip_stream_t stream);
 }  // namespace lapis

@@ -206,7 +206,7 @@ template <typename T, int CH, int WAVES, bool VEC, bool NT>
 __global__ __launch_bounds__(64 * WAVES) void spmv_nnzsplit_kernel(
     int nrows, int nnz, int nchunks, const int *__restrict__ pos, const int *__restrict__ crd,
     const T *__restrict__ val, const T *__restrict__ x, T *__restrict__ y,
-    const int *__restrict__ chunk_row, T *__restrict__ part_first, T *__restrict__ part_last) {
+    const int *__restrict__ chunk_row, T *__restrict__ part_first, T *__restrict__ part_last, int accumulate) {
   __shared__ T lds[WAVES * CH];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -236,7 +236,7 @@ __global__ __launch_bounds__(64 * WAVES) void spmv_nnzsplit_kernel(
       const bool starts = ps >= e0;
       const bool ends = pe <= e1;
       if (starts && ends)
-        y[r] = acc + y[r];
+        y[r] = accumulate ? acc + y[r] : acc;
       else if (!starts)
         part_first[c] = acc;
       else
@@ -252,7 +252,7 @@ __global__ __launch_bounds__(64 * WAVES) void spmv_nnzsplit_kernel(
 template <typename T, int CH>
 __global__ __launch_bounds__(256) void spmv_nnzsplit_fixup_kernel(
     int nchunks, const int *__restrict__ pos, const int *__restrict__ chunk_row,
-    const T *__restrict__ part_first, const T *__restrict__ part_last, T *__restrict__ y) {
+    const T *__restrict__ part_first, const T *__restrict__ part_last, T *__restrict__ y, int accumulate) {
   const int lane = threadIdx.x & 63;
   const long long c = (long long)blockIdx.x * 256 + threadIdx.x + 1;
   bool owner = false;
@@ -284,7 +284,7 @@ __global__ __launch_bounds__(256) void spmv_nnzsplit_fixup_kernel(
     part = group_sum<64>(part);
     if (lane == src) total = part_last[cfirst - 1] + part;
   }
-  if (owner) y[r] = total + y[r];
+  if (owner) y[r] = accumulate ? total + y[r] : total;
 }
 
 // ------------------------------------------------------------------------------
@@ -474,18 +474,18 @@ int launch_rowblock(int64_t nrows, int64_t nnz, const int *pos, const int *crd, 
 
 template <typename T, bool VEC, bool NT>
 int launch_nnzsplit(const lapis_hip_csr_plan *p, const int *pos, const int *crd, const T *val, const T *x,
-                    T *y, hipStream_t st) {
+                    T *y, hipStream_t st, int accumulate = 1) {
   const int nchunks = p->nchunks;
   const int blocks = (int)ceil_div(nchunks, kWavesPerBlock);
   launch_timed(spmv_nnzsplit_kernel<T, kChunk, kWavesPerBlock, VEC, NT>, dim3(blocks), dim3(64 * kWavesPerBlock),
                st, (int)p->stats.nrows, (int)p->stats.nnz, nchunks, pos, crd, val, x, y,
-               (const int *)p->chunk_row, static_cast<T *>(p->part_first), static_cast<T *>(p->part_last));
+               (const int *)p->chunk_row, static_cast<T *>(p->part_first), static_cast<T *>(p->part_last), accumulate);
   LAPIS_LAUNCH_CHECK();
   if (nchunks > 1) {
     const int fblocks = (int)ceil_div(nchunks - 1, 256);
     hipLaunchKernelGGL((spmv_nnzsplit_fixup_kernel<T, kChunk>), dim3(fblocks), dim3(256), 0, st, nchunks, pos,
                        p->chunk_row, static_cast<const T *>(p->part_first),
-                       static_cast<const T *>(p->part_last), y);
+                       static_cast<const T *>(p->part_last), y, accumulate);
     LAPIS_LAUNCH_CHECK();
   }
   return LAPIS_HIP_OK;
@@ -551,6 +551,29 @@ int spmv_impl(lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, const int3
   }
 }
 
+}  // namespace
+
+namespace lapis {
+// y = A x (y is not read).  The row-split kernel writes every non-empty row itself;
+// any other case zero-fills y and accumulates.
+int spmv_overwrite_f64(lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, const int32_t *pos,
+                       const int32_t *crd, const double *val, const double *x, double *y,
+                       lapis_hip_stream_t stream) {
+  if (plan && plan->stats.kernel == LAPIS_HIP_SPMV_NNZSPLIT && plan->stats.empty_rows == 0 && plan->stats.nnz > 0 &&
+      plan->stats.nrows == nrows && plan->stats.ncols == ncols && plan->pos == pos && aligned16(crd) &&
+      aligned16(val)) {
+    LAPIS_CHECK_INIT();
+    hipStream_t st = as_stream(stream);
+    return plan->nontemporal ? launch_nnzsplit<double, true, true>(plan, pos, crd, val, x, y, st, 0)
+                             : launch_nnzsplit<double, true, false>(plan, pos, crd, val, x, y, st, 0);
+  }
+  const int rc = lapis_hip_fill_f64(nrows, 0.0, y, stream);
+  if (rc != LAPIS_HIP_OK) return rc;
+  return lapis_hip_spmv_csr_f64_i32(plan, nrows, ncols, pos, crd, val, x, y, stream);
+}
+}  // namespace lapis
+
+namespace {
 void free_plan_buffers(lapis_hip_csr_plan *p) {
   if (p->chunk_row) (void)hipFree(p->chunk_row);
   if (p->part_first) (void)hipFree(p->part_first);
