@@ -100,10 +100,12 @@ struct ScaleOp {
 };
 
 // ---- dot --------------------------------------------------------------------------
-// Stage 1: each block sums a grid-strided slice (per-thread partial, DPP wave sum,
-// LDS across the waves in wave order) into partials[block].  The block that takes
-// the last ticket sums partials[] in index order and writes init + total, so the
-// result is the same from run to run.
+// Two launches: each block sums a grid-strided slice (per-thread partial, DPP wave
+// sum, LDS across the four waves in wave order) into partials[block]; a one-block
+// kernel behind it adds the partials in index order and writes init + total.  The
+// order is fixed, so the result is the same from run to run, and the kernel boundary
+// does the ordering: no device-scope fence, which on a multi-XCD part would write
+// back and invalidate L2 once per block.
 template <typename T>
 __device__ __forceinline__ T block_sum_256(T v, T *lds4) {
   v = group_sum<64>(v);
@@ -116,31 +118,33 @@ __device__ __forceinline__ T block_sum_256(T v, T *lds4) {
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void dot_kernel(long long n, const T *__restrict__ x, const T *__restrict__ y,
-                                                  T init, T *partials, unsigned *ticket,
-                                                  T *__restrict__ result) {
+__global__ __launch_bounds__(256) void dot_partial_kernel(long long n, const T *__restrict__ x,
+                                                          const T *__restrict__ y, T *__restrict__ partials,
+                                                          int vec) {
+  typedef typename VecOf<T>::type V;
+  constexpr int VW = VecOf<T>::width;
   __shared__ T lds4[4];
-  __shared__ bool is_last;
   T acc = T(0);
-  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
+  const long long nv = vec ? n / VW : 0;  // 128-bit accesses when both vectors are 16-byte aligned
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < nv; i += (long long)gridDim.x * 256) {
+    const V a = reinterpret_cast<const V *>(x)[i], b = reinterpret_cast<const V *>(y)[i];
+#pragma unroll
+    for (int e = 0; e < VW; ++e) acc = acc + a[e] * b[e];
+  }
+  for (long long i = nv * VW + (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
     acc = acc + x[i] * y[i];
   const T total = block_sum_256(acc, lds4);
-  if (threadIdx.x == 0) {
-    partials[blockIdx.x] = total;
-    __threadfence();
-    const unsigned t = atomicAdd(ticket, 1u);
-    is_last = (t == gridDim.x - 1);
-  }
-  __syncthreads();
-  if (!is_last) return;
-  __threadfence();
+  if (threadIdx.x == 0) partials[blockIdx.x] = total;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void dot_final_kernel(int count, const T *__restrict__ partials, T init,
+                                                        T *__restrict__ result) {
+  __shared__ T lds4[4];
   T s = T(0);
-  for (unsigned i = threadIdx.x; i < gridDim.x; i += 256) s = s + partials[i];
+  for (int i = threadIdx.x; i < count; i += 256) s = s + partials[i];
   const T all = block_sum_256(s, lds4);
-  if (threadIdx.x == 0) {
-    *result = all + init;
-    *ticket = 0u;
-  }
+  if (threadIdx.x == 0) *result = all + init;
 }
 
 int dot_grid(int64_t n) {
@@ -150,17 +154,16 @@ int dot_grid(int64_t n) {
 }
 
 template <typename T>
-int launch_dot(int64_t n, const T *x, const T *y, T init, T *result, T *partials, unsigned *ticket,
-               hipStream_t st) {
-  hipLaunchKernelGGL((dot_kernel<T>), dim3(dot_grid(n)), dim3(256), 0, st, (long long)n, x, y, init, partials,
-                     ticket, result);
+int launch_dot(int64_t n, const T *x, const T *y, T init, T *result, T *partials, hipStream_t st) {
+  const int grid = dot_grid(n);
+  hipLaunchKernelGGL((dot_partial_kernel<T>), dim3(grid), dim3(256), 0, st, (long long)n, x, y, partials,
+                     (aligned16(x) && aligned16(y)) ? 1 : 0);
+  hipLaunchKernelGGL((dot_final_kernel<T>), dim3(1), dim3(256), 0, st, grid, (const T *)partials, init, result);
   LAPIS_LAUNCH_CHECK();
   return LAPIS_HIP_OK;
 }
-template int launch_dot<double>(int64_t, const double *, const double *, double, double *, double *, unsigned *,
-                                hipStream_t);
-template int launch_dot<float>(int64_t, const float *, const float *, float, float *, float *, unsigned *,
-                               hipStream_t);
+template int launch_dot<double>(int64_t, const double *, const double *, double, double *, double *, hipStream_t);
+template int launch_dot<float>(int64_t, const float *, const float *, float, float *, float *, hipStream_t);
 
 // Scratch for the stand-alone dot entry points: a ring of slots, one per call, so
 // that dots queued on different streams do not share partials unless more than
@@ -168,19 +171,14 @@ template int launch_dot<float>(int64_t, const float *, const float *, float, flo
 namespace {
 constexpr int kSlots = 64;
 std::mutex g_scratch_mutex;
-char *g_scratch = nullptr;  // kSlots * (kDotMaxBlocks * 8 + 256) bytes
+char *g_scratch = nullptr;  // kSlots * kDotMaxBlocks * 8 bytes
 unsigned g_next_slot = 0;
-constexpr size_t kSlotBytes = (size_t)kDotMaxBlocks * 8 + 256;
+constexpr size_t kSlotBytes = (size_t)kDotMaxBlocks * 8;
 
-int take_slot(void **partials, unsigned **ticket) {
+int take_slot(void **partials) {
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
-  if (!g_scratch) {
-    LAPIS_HIP_TRY(hipMalloc(&g_scratch, kSlots * kSlotBytes));
-    LAPIS_HIP_TRY(hipMemset(g_scratch, 0, kSlots * kSlotBytes));
-  }
-  char *slot = g_scratch + (size_t)(g_next_slot++ % kSlots) * kSlotBytes;
-  *partials = slot;
-  *ticket = reinterpret_cast<unsigned *>(slot + (size_t)kDotMaxBlocks * 8);
+  if (!g_scratch) LAPIS_HIP_TRY(hipMalloc(&g_scratch, kSlots * kSlotBytes));
+  *partials = g_scratch + (size_t)(g_next_slot++ % kSlots) * kSlotBytes;
   return LAPIS_HIP_OK;
 }
 
@@ -191,10 +189,9 @@ int dot_entry(const char *what, int64_t n, const T *x, const T *y, T init, T *re
   LAPIS_REQUIRE(result, "%s: null result", what);
   LAPIS_REQUIRE(n == 0 || (x && y), "%s: null vector with n=%lld", what, (long long)n);
   void *partials = nullptr;
-  unsigned *ticket = nullptr;
-  const int rc = take_slot(&partials, &ticket);
+  const int rc = take_slot(&partials);
   if (rc != LAPIS_HIP_OK) return rc;
-  return launch_dot<T>(n, x, y, init, result, static_cast<T *>(partials), ticket, as_stream(stream));
+  return launch_dot<T>(n, x, y, init, result, static_cast<T *>(partials), as_stream(stream));
 }
 }  // namespace
 

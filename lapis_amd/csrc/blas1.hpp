@@ -11,10 +11,8 @@ constexpr int kDotMaxBlocks = 2048;  // upper bound of dot_grid(); sizes the par
 // Number of blocks (= partial sums) a dot over n elements uses.
 int dot_grid(int64_t n);
 
-// *result = init + sum x[i]*y[i].  `partials` holds kDotMaxBlocks elements of T,
-// `*ticket` must be 0 on entry and is 0 again on exit.
+// *result = init + sum x[i]*y[i].  `partials` holds kDotMaxBlocks elements of T.
 template <typename T>
-int launch_dot(int64_t n, const T *x, const T *y, T init, T *result, T *partials, unsigned *ticket,
-               hipStream_t st);
+int launch_dot(int64_t n, const T *x, const T *y, T init, T *result, T *partials, hipStream_t st);
 
 }  // namespace lapis

@@ -8,6 +8,12 @@
 //   z = r*dinv ; rz' = r.z ; beta = rz'/rz ; p = 1*z + beta*p ; i = i+1
 // r.z at the top of an iteration is the rz' of the one before (same vectors), so
 // it is carried instead of recomputed; without a preconditioner z is r and rz' is rr.
+//
+// Every dot product is two launches: the vector kernel leaves one partial per block,
+// a one-block kernel behind it adds the partials in index order and updates the
+// scalars.  Kernel boundaries order the two, so no block ever needs a device-scope
+// fence (on a multi-XCD part such a fence writes back and invalidates L2, and two
+// thousand of them per kernel cost more than the vector pass itself).
 #include <algorithm>
 #include <cmath>
 
@@ -28,7 +34,7 @@ struct CgState {
   unsigned long long maxiter;
   double tol;
   int done;
-  unsigned ticket[3];
+  int roll_pending;  // update_p has run: rz = rz_next and i = i+1 are due
 };
 
 __device__ __forceinline__ double block_sum_256d(double v, double *lds4) {
@@ -40,36 +46,30 @@ __device__ __forceinline__ double block_sum_256d(double v, double *lds4) {
   return total;
 }
 
-// Publishes this block's partial and tells whether this block is the last to do so;
-// the last block then owns the ordered final sum.
-__device__ __forceinline__ bool publish_partial(double v, double *partials, unsigned *ticket, bool *flag) {
-  if (threadIdx.x == 0) {
-    partials[blockIdx.x] = v;
-    __threadfence();
-    *flag = (atomicAdd(ticket, 1u) == gridDim.x - 1);
-  }
-  __syncthreads();
-  const bool last = *flag;
-  if (last) __threadfence();
-  return last;
-}
-
-__device__ __forceinline__ double ordered_total(const double *partials, double *lds4) {
+// Sum of partials[0..count) in a fixed order, by one block of 256 threads.
+__device__ __forceinline__ double ordered_total(const double *partials, int count, double *lds4) {
   double s = 0.0;
-  for (unsigned i = threadIdx.x; i < gridDim.x; i += 256) s = s + partials[i];
+  for (int i = threadIdx.x; i < count; i += 256) s = s + partials[i];
   return block_sum_256d(s, lds4);
 }
 
-// r0 = b, z0 = r0*dinv (or r0), p0 = z0, x0 = 0; partial sums of r0.r0 and r0.z0.
+// The vector passes below walk their arrays two doubles (one 128-bit access) per
+// thread and trip when every array is 16-byte aligned (`vec`), element by element
+// otherwise; an odd last element is taken by the scalar tail.
+#define CG_GRID_STRIDE(i, first, count) \
+  for (long long i = (first) + (long long)blockIdx.x * 256 + threadIdx.x; i < (count); i += (long long)gridDim.x * 256)
+
+__device__ __forceinline__ v2d ld2(const double *p, long long i) { return reinterpret_cast<const v2d *>(p)[i]; }
+__device__ __forceinline__ void st2(double *p, long long i, v2d v) { reinterpret_cast<v2d *>(p)[i] = v; }
+
+// r0 = b, z0 = r0*dinv (or r0), p0 = z0, x0 = 0; block partials of r0.r0 and r0.z0.
 __global__ __launch_bounds__(256) void cg_init_kernel(long long n, const double *__restrict__ b,
                                                       const double *__restrict__ dinv, double *__restrict__ x,
                                                       double *__restrict__ r, double *__restrict__ z,
-                                                      double *__restrict__ p, CgState *st,
-                                                      double *__restrict__ partials) {
+                                                      double *__restrict__ p, double *__restrict__ partials) {
   __shared__ double lds4[4];
-  __shared__ bool flag;
   double rr = 0.0, rz = 0.0;
-  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) {
+  CG_GRID_STRIDE(i, 0, n) {
     const double ri = b[i];
     const double zi = dinv ? ri * dinv[i] : ri;
     r[i] = ri;
@@ -81,49 +81,53 @@ __global__ __launch_bounds__(256) void cg_init_kernel(long long n, const double 
   }
   const double brr = block_sum_256d(rr, lds4);
   const double brz = block_sum_256d(rz, lds4);
-  if (threadIdx.x == 0) partials[kDotMaxBlocks + blockIdx.x] = brz;
-  if (!publish_partial(brr, partials, &st->ticket[0], &flag)) return;
-  const double trr = ordered_total(partials, lds4);
-  const double trz = ordered_total(partials + kDotMaxBlocks, lds4);
   if (threadIdx.x == 0) {
-    st->initres = sqrt(trr);
-    st->rz = trz;
-    st->iter = 1;
-    st->done = 0;
-    st->ticket[0] = 0u;
+    partials[blockIdx.x] = brr;
+    partials[kDotMaxBlocks + blockIdx.x] = brz;
   }
 }
 
-// pAp = p . Ap
+// block partials of p . Ap
 __global__ __launch_bounds__(256) void cg_pap_kernel(long long n, const double *__restrict__ p,
-                                                     const double *__restrict__ Ap, CgState *st,
-                                                     double *__restrict__ partials) {
+                                                     const double *__restrict__ Ap, double *__restrict__ partials,
+                                                     int vec) {
   __shared__ double lds4[4];
-  __shared__ bool flag;
   double acc = 0.0;
-  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256)
-    acc = acc + p[i] * Ap[i];
-  const double bsum = block_sum_256d(acc, lds4);
-  if (!publish_partial(bsum, partials, &st->ticket[0], &flag)) return;
-  const double total = ordered_total(partials, lds4);
-  if (threadIdx.x == 0) {
-    st->pAp = total;
-    st->ticket[0] = 0u;
+  const long long nv = vec ? n / 2 : 0;
+  CG_GRID_STRIDE(i, 0, nv) {
+    const v2d a = ld2(p, i), b = ld2(Ap, i);
+    acc = acc + a.x * b.x;
+    acc = acc + a.y * b.y;
   }
+  CG_GRID_STRIDE(i, 2 * nv, n) acc = acc + p[i] * Ap[i];
+  const double bsum = block_sum_256d(acc, lds4);
+  if (threadIdx.x == 0) partials[blockIdx.x] = bsum;
 }
 
-// x += alpha p ; r -= alpha Ap ; rr = r.r ; the last block decides convergence.
+// x += alpha p ; r -= alpha Ap ; block partials of r.r
 __global__ __launch_bounds__(256) void cg_update_xr_kernel(long long n, const double *__restrict__ p,
                                                            const double *__restrict__ Ap, double *__restrict__ x,
-                                                           double *__restrict__ r, CgState *st,
-                                                           double *__restrict__ partials, int preconditioned) {
+                                                           double *__restrict__ r, const CgState *st,
+                                                           double *__restrict__ partials, int vec) {
   __shared__ double lds4[4];
-  __shared__ bool flag;
   if (st->done) return;
   const double alpha = st->rz / st->pAp;
   const double malpha = -alpha;
   double rr = 0.0;
-  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) {
+  const long long nv = vec ? n / 2 : 0;
+  CG_GRID_STRIDE(i, 0, nv) {
+    const v2d pv = ld2(p, i), av = ld2(Ap, i);
+    v2d xv = ld2(x, i), rv = ld2(r, i);
+    xv.x = xv.x + pv.x * alpha;
+    xv.y = xv.y + pv.y * alpha;
+    rv.x = rv.x + av.x * malpha;
+    rv.y = rv.y + av.y * malpha;
+    st2(x, i, xv);
+    st2(r, i, rv);
+    rr = rr + rv.x * rv.x;
+    rr = rr + rv.y * rv.y;
+  }
+  CG_GRID_STRIDE(i, 2 * nv, n) {
     const double xt = p[i] * alpha;
     const double xi = x[i] + xt;
     const double rt = Ap[i] * malpha;
@@ -133,59 +137,98 @@ __global__ __launch_bounds__(256) void cg_update_xr_kernel(long long n, const do
     rr = rr + ri * ri;
   }
   const double bsum = block_sum_256d(rr, lds4);
-  if (!publish_partial(bsum, partials, &st->ticket[1], &flag)) return;
-  const double total = ordered_total(partials, lds4);
-  if (threadIdx.x == 0) {
-    const double relres = sqrt(total) / st->initres;
-    st->rr = total;
-    st->relres = relres;
-    if (!preconditioned) st->rz_next = total;
-    const bool go_on = (relres > st->tol) && (st->iter != st->maxiter);
-    if (!go_on) st->done = 1;
-    st->ticket[1] = 0u;
-  }
+  if (threadIdx.x == 0) partials[blockIdx.x] = bsum;
 }
 
-// z = r * dinv ; rz_next = r.z     (preconditioned runs only)
+// z = r * dinv ; block partials of r.z     (preconditioned runs only)
 __global__ __launch_bounds__(256) void cg_precond_kernel(long long n, const double *__restrict__ r,
                                                          const double *__restrict__ dinv, double *__restrict__ z,
-                                                         CgState *st, double *__restrict__ partials) {
+                                                         const CgState *st, double *__restrict__ partials, int vec) {
   __shared__ double lds4[4];
-  __shared__ bool flag;
   if (st->done) return;
   double acc = 0.0;
-  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) {
+  const long long nv = vec ? n / 2 : 0;
+  CG_GRID_STRIDE(i, 0, nv) {
+    const v2d rv = ld2(r, i), dv = ld2(dinv, i);
+    v2d zv;
+    zv.x = rv.x * dv.x;
+    zv.y = rv.y * dv.y;
+    st2(z, i, zv);
+    acc = acc + rv.x * zv.x;
+    acc = acc + rv.y * zv.y;
+  }
+  CG_GRID_STRIDE(i, 2 * nv, n) {
     const double ri = r[i];
     const double zi = ri * dinv[i];
     z[i] = zi;
     acc = acc + ri * zi;
   }
   const double bsum = block_sum_256d(acc, lds4);
-  if (!publish_partial(bsum, partials, &st->ticket[2], &flag)) return;
-  const double total = ordered_total(partials, lds4);
-  if (threadIdx.x == 0) {
-    st->rz_next = total;
-    st->ticket[2] = 0u;
-  }
+  if (threadIdx.x == 0) partials[blockIdx.x] = bsum;
 }
 
-// p = z + beta p with beta = rz_next/rz.  The scalars are rolled forward
-// (rz = rz_next, i = i+1) by a separate one-thread kernel queued behind this one, so
-// that every block of this kernel still reads the pair it needs.
+// p = z + beta p with beta = rz_next/rz.
 __global__ __launch_bounds__(256) void cg_update_p_kernel(long long n, const double *__restrict__ z,
-                                                          double *__restrict__ p, const CgState *st) {
+                                                          double *__restrict__ p, const CgState *st, int vec) {
   if (st->done) return;
   const double beta = st->rz_next / st->rz;
-  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) {
+  const long long nv = vec ? n / 2 : 0;
+  CG_GRID_STRIDE(i, 0, nv) {
+    const v2d zv = ld2(z, i);
+    v2d pv = ld2(p, i);
+    pv.x = zv.x + pv.x * beta;
+    pv.y = zv.y + pv.y * beta;
+    st2(p, i, pv);
+  }
+  CG_GRID_STRIDE(i, 2 * nv, n) {
     const double pt = p[i] * beta;
     p[i] = z[i] + pt;
   }
 }
 
-__global__ void cg_roll_kernel(CgState *st) {
+// The one-block kernels that turn block partials into scalars.
+enum { kStageInit = 0, kStagePap = 1, kStageResidual = 2, kStagePrecond = 3 };
+
+__global__ __launch_bounds__(256) void cg_scalar_kernel(int stage, int count, const double *__restrict__ partials,
+                                                        CgState *st, int preconditioned) {
+  __shared__ double lds4[4];
+  if (stage == kStageInit) {
+    const double trr = ordered_total(partials, count, lds4);
+    const double trz = ordered_total(partials + kDotMaxBlocks, count, lds4);
+    if (threadIdx.x == 0) {
+      st->initres = sqrt(trr);
+      st->rz = trz;
+      st->iter = 1;
+      st->done = 0;
+      st->roll_pending = 0;
+    }
+    return;
+  }
   if (st->done) return;
-  st->rz = st->rz_next;
-  st->iter = st->iter + 1;
+  const double total = ordered_total(partials, count, lds4);
+  if (threadIdx.x != 0) return;
+  if (stage == kStagePap) {
+    // the first scalar step of an iteration also rolls the previous one forward:
+    // update_p of that iteration has read rz and rz_next by now
+    if (st->roll_pending) {
+      st->rz = st->rz_next;
+      st->iter = st->iter + 1;
+      st->roll_pending = 0;
+    }
+    st->pAp = total;
+  } else if (stage == kStageResidual) {
+    const double relres = sqrt(total) / st->initres;
+    st->rr = total;
+    st->relres = relres;
+    if (!preconditioned) st->rz_next = total;
+    const bool go_on = (relres > st->tol) && (st->iter != st->maxiter);
+    if (go_on)
+      st->roll_pending = 1;
+    else
+      st->done = 1;
+  } else {
+    st->rz_next = total;
+  }
 }
 
 }  // namespace lapis
@@ -211,6 +254,7 @@ extern "C" int lapis_hip_pcg_f64_i32(lapis_hip_csr_plan *plan, int64_t n, const 
   int rc = LAPIS_HIP_OK;
   lapis_hip_csr_plan *own_plan = nullptr;
   double *own_work = nullptr;
+  int64_t stride = n;  // distance between the four work vectors
   CgState *state = nullptr;
   double *partials = nullptr;
   bool finished = false;
@@ -247,10 +291,12 @@ extern "C" int lapis_hip_pcg_f64_i32(lapis_hip_csr_plan *plan, int64_t n, const 
     plan = own_plan;
   }
   if (!work) {
-    PCG_TRY(hipMalloc(&own_work, sizeof(double) * 4 * (size_t)n));
+    // own scratch: an even stride keeps all four vectors 16-byte aligned
+    stride = (n + 1) & ~(int64_t)1;
+    PCG_TRY(hipMalloc(&own_work, sizeof(double) * 4 * (size_t)stride));
     work = own_work;
   }
-  double *r = work, *z = dinv ? work + n : work, *p = work + 2 * n, *Ap = work + 3 * n;
+  double *r = work, *z = dinv ? work + stride : work, *p = work + 2 * stride, *Ap = work + 3 * stride;
   PCG_TRY(hipMalloc(&state, sizeof(CgState)));
   PCG_TRY(hipMalloc(&partials, sizeof(double) * 2 * kDotMaxBlocks));
   CgState h{};
@@ -260,8 +306,12 @@ extern "C" int lapis_hip_pcg_f64_i32(lapis_hip_csr_plan *plan, int64_t n, const 
 
   const int grid = dot_grid(n);
   const int pre = dinv ? 1 : 0;
-  hipLaunchKernelGGL(cg_init_kernel, dim3(grid), dim3(256), 0, st, (long long)n, b, dinv, x, r, z, p, state,
-                     partials);
+  const int vec = (aligned16(x) && aligned16(r) && aligned16(z) && aligned16(p) && aligned16(Ap) &&
+                   (!dinv || aligned16(dinv)))
+                      ? 1
+                      : 0;
+  hipLaunchKernelGGL(cg_init_kernel, dim3(grid), dim3(256), 0, st, (long long)n, b, dinv, x, r, z, p, partials);
+  hipLaunchKernelGGL(cg_scalar_kernel, dim3(1), dim3(256), 0, st, (int)kStageInit, grid, partials, state, pre);
   PCG_TRY(hipGetLastError());
 
   // The host looks at the device's `done` flag after each batch of iterations; a
@@ -285,14 +335,19 @@ extern "C" int lapis_hip_pcg_f64_i32(lapis_hip_csr_plan *plan, int64_t n, const 
     for (int it = 0; it < todo; ++it) {
       // Ap = A p: the reference zero-fills Ap and accumulates (examples/pcg_solve.py:12-19)
       PCG_RC(spmv_overwrite_f64(plan, n, n, pos, crd, val, p, Ap, stream));
-      hipLaunchKernelGGL(cg_pap_kernel, dim3(grid), dim3(256), 0, st, (long long)n, p, Ap, state, partials);
+      hipLaunchKernelGGL(cg_pap_kernel, dim3(grid), dim3(256), 0, st, (long long)n, p, Ap, partials, vec);
+      hipLaunchKernelGGL(cg_scalar_kernel, dim3(1), dim3(256), 0, st, (int)kStagePap, grid, partials, state, pre);
       hipLaunchKernelGGL(cg_update_xr_kernel, dim3(grid), dim3(256), 0, st, (long long)n, p, Ap, x, r, state,
-                         partials, pre);
-      if (pre)
+                         partials, vec);
+      hipLaunchKernelGGL(cg_scalar_kernel, dim3(1), dim3(256), 0, st, (int)kStageResidual, grid, partials, state,
+                         pre);
+      if (pre) {
         hipLaunchKernelGGL(cg_precond_kernel, dim3(grid), dim3(256), 0, st, (long long)n, r, dinv, z, state,
-                           partials);
-      hipLaunchKernelGGL(cg_update_p_kernel, dim3(grid), dim3(256), 0, st, (long long)n, z, p, state);
-      hipLaunchKernelGGL(cg_roll_kernel, dim3(1), dim3(1), 0, st, state);
+                           partials, vec);
+        hipLaunchKernelGGL(cg_scalar_kernel, dim3(1), dim3(256), 0, st, (int)kStagePrecond, grid, partials, state,
+                           pre);
+      }
+      hipLaunchKernelGGL(cg_update_p_kernel, dim3(grid), dim3(256), 0, st, (long long)n, z, p, state, vec);
       PCG_TRY(hipGetLastError());
     }
     launched += (uint64_t)todo;

@@ -3,6 +3,8 @@
 // device, one warm-up call, then `trials` calls each followed by a fence, print the
 // mean time.  Usage: lapis_spmv_bench matrix.mtx [trials=1000] [kernel]
 //   kernel: auto (default) | reference | subwarpN | rowblock | nnzsplit | colblock
+// Instead of a file, `gen:laplace3d:N` builds the 7-point Laplacian on an N^3 grid
+// (N = 100 is the size of the reference's Laplace3D_100).
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -114,6 +116,32 @@ bool read_matrix_market(const std::string &path, Csr &A, std::string &err) {
   return true;
 }
 
+// 7-point Laplacian on an n^3 grid, x fastest, diagonal 6 and off-diagonals -1.
+void laplace3d(int n, Csr &A) {
+  const int64_t N = (int64_t)n * n * n;
+  A.nrows = A.ncols = N;
+  A.pos.assign((size_t)N + 1, 0);
+  A.crd.clear();
+  A.val.clear();
+  A.crd.reserve((size_t)N * 7);
+  A.val.reserve((size_t)N * 7);
+  for (int64_t i = 0; i < N; ++i) {
+    const int ix = (int)(i % n), iy = (int)((i / n) % n), iz = (int)(i / ((int64_t)n * n));
+    auto put = [&](int64_t c, double v) {
+      A.crd.push_back((int32_t)c);
+      A.val.push_back(v);
+    };
+    if (iz > 0) put(i - (int64_t)n * n, -1);
+    if (iy > 0) put(i - n, -1);
+    if (ix > 0) put(i - 1, -1);
+    put(i, 6);
+    if (ix < n - 1) put(i + 1, -1);
+    if (iy < n - 1) put(i + n, -1);
+    if (iz < n - 1) put(i + (int64_t)n * n, -1);
+    A.pos[(size_t)i + 1] = (int32_t)A.crd.size();
+  }
+}
+
 #define CHECK_HIP(expr)                                                              \
   do {                                                                               \
     hipError_t e_ = (expr);                                                          \
@@ -142,12 +170,22 @@ int main(int argc, const char **argv) {
   const int trials = argc > 2 ? std::max(1, atoi(argv[2])) : 1000;
   const std::string kernel = argc > 3 ? argv[3] : "auto";
   CHECK_LAPIS(lapis_hip_init());
-  std::cout << "Reading matrix from " << mfile << "...\n";
   Csr A;
   std::string err;
-  if (!read_matrix_market(mfile, A, err)) {
-    std::cerr << "error: " << err << "\n";
-    return 1;
+  if (mfile.rfind("gen:laplace3d:", 0) == 0) {
+    const int n = atoi(mfile.c_str() + 14);
+    if (n < 1 || n > 1000) {
+      std::cerr << "error: grid size outside [1, 1000]\n";
+      return 1;
+    }
+    std::cout << "Generating the 7-point Laplacian on a " << n << "^3 grid...\n";
+    laplace3d(n, A);
+  } else {
+    std::cout << "Reading matrix from " << mfile << "...\n";
+    if (!read_matrix_market(mfile, A, err)) {
+      std::cerr << "error: " << err << "\n";
+      return 1;
+    }
   }
   const int64_t nnz = (int64_t)A.crd.size();
   std::cout << "Read matrix (" << A.nrows << "x" << A.ncols << " with " << nnz << " entries)\n";

@@ -131,13 +131,17 @@ def test_plan_statistics_and_reference_decision(gpu, oracle):
     hint = oracle.csr_parallelism_hint(A.pos)
     assert hint in (16, 17) and s["reference_hint"] == hint
     assert s["reference_vector_length"] == oracle.thread_parallel_vector_length(hint, 64) == 4
-    assert s["kernel_name"] == "nnzsplit"
+    assert s["kernel_name"] == "rowblock"  # about a million non-zeros: one launch beats two
+    assert s["mean_chunk_col_span"] > 0.9 * A.ncols and s["colblock_recommended"] == 0
     B, _ = gen.config3(scale=1 / 16)
     sb = gpu.CsrPlan(B.nrows, B.ncols, dev(B.pos), dev(B.crd), value_bytes=4).stats()
     assert sb["kernel_name"] == "nnzsplit" and sb["reference_vector_length"] == 8
-    C = gen.poisson_random(2000, 300.0, seed=3)
+    C = gen.poisson_random(6000, 2400.0, seed=3)
     sc = gpu.CsrPlan(C.nrows, C.ncols, dev(C.pos), dev(C.crd)).stats()
     assert sc["kernel_name"] == "subwarp" and sc["width"] == 64
+    D, _ = gen.config5(scale=(110 / 192) ** 3)
+    sd = gpu.CsrPlan(D.nrows, D.ncols, dev(D.pos), dev(D.crd)).stats()
+    assert sd["kernel_name"] == "nnzsplit" and sd["mean_chunk_col_span"] < 3 * 110 * 110
 
 
 def test_unaligned_buffers_take_the_scalar_path(gpu, oracle):
