@@ -165,6 +165,12 @@ int lapis_hip_spmm_csr_f64_i32(int64_t nrows, int64_t ncols, int64_t k, const in
                                const int32_t *crd, const double *val, const double *B, int64_t ldb,
                                double *C, int64_t ldc, lapis_hip_stream_t stream);
 
+/* Batched CSRV product of examples/bspmm.py:22-50 (out(n1,dh,nh) += A(n1,n2,nh) * V(n2,dh,nh)):
+ * A is CSR over (n1, n2), each non-zero carries nh values (val has nnz*nh entries). */
+int lapis_hip_bspmm_csrv_f32_i32(int64_t n1, int64_t n2, int64_t dh, int64_t nh, const int32_t *pos,
+                                 const int32_t *crd, const float *val, const float *V, float *out,
+                                 lapis_hip_stream_t stream);
+
 /* ---- dense vector kernels of CG -------------------------------------------- */
 
 /* *result = init + sum_i x[i]*y[i]; `result` is a DEVICE scalar (no host sync,
@@ -209,6 +215,24 @@ int lapis_hip_pcg_f64_i32(lapis_hip_csr_plan *plan, int64_t n, const int32_t *po
                           const double *val, const double *b, const double *dinv, double tol,
                           uint64_t maxiter, double *x, uint64_t *iters, double *relres, double *work,
                           lapis_hip_stream_t stream);
+
+/* The solver variant of examples/hitting_times.py:97-149: the operator is the masked
+ * normalized graph Laplacian plpt (:73-93), y = mask*(d*(mask*p) - A (mask*p)), and
+ * the preconditioner is an elementwise division by d.  `work` is 5*n doubles or NULL. */
+int lapis_hip_pcg_masked_f64_i32(lapis_hip_csr_plan *plan, int64_t n, const int32_t *pos, const int32_t *crd,
+                                 const double *val, const double *b, const double *mask, const double *d,
+                                 double tol, uint64_t maxiter, double *x, uint64_t *iters, double *relres,
+                                 double *work, lapis_hip_stream_t stream);
+
+/* func @mht of examples/hitting_times.py:153-179: scales val by alpha IN PLACE
+ * (scale_csr, :51-71), then two masked CG solves for the first two hitting-time
+ * moments.  Synchronises `stream`. */
+int lapis_hip_mht_f64_i32(lapis_hip_csr_plan *plan, int64_t n, int64_t nnz, const int32_t *pos,
+                          const int32_t *crd, double *val, const double *mask, const double *d, double alpha,
+                          double tol, uint64_t maxiter, double *mom1, double *mom2, lapis_hip_stream_t stream);
+/* func @normalize_mom2 of examples/hitting_times.py:181-198: out = sqrt(mom2 - mom1*mom1). */
+int lapis_hip_normalize_mom2_f64(int64_t n, const double *mom1, const double *mom2, double *out,
+                                 lapis_hip_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -95,6 +95,13 @@ void py_spmm_f64(lapis_memref_2d_f64 **ret0, lapis_memref_1d_i32 *pos, lapis_mem
 /* func @plus_norm(x, y) -> (x+y, ||x+y||) of examples/multiple_results.py:8-19. */
 void py_plus_norm(lapis_memref_1d_f64 **ret0, double *ret1, lapis_memref_1d_f64 *x, lapis_memref_1d_f64 *y);
 
+/* func @mht(A, mask, d, alpha, tol, maxiter) -> (mom1, mom2) and
+ * func @normalize_mom2(mom1, mom2) -> stdev of examples/hitting_times.py:153-198. */
+void py_mht(lapis_memref_1d_f64 **ret0, lapis_memref_1d_f64 **ret1, lapis_memref_1d_i32 *pos,
+            lapis_memref_1d_i32 *crd, lapis_memref_1d_f64 *val, const lapis_csr_specifier *spec,
+            lapis_memref_1d_f64 *mask, lapis_memref_1d_f64 *d, double alpha, double tol, size_t maxiter);
+void py_normalize_mom2(lapis_memref_1d_f64 **ret0, lapis_memref_1d_f64 *mom1, lapis_memref_1d_f64 *mom2);
+
 #ifdef __cplusplus
 }
 #endif

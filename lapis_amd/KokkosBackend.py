@@ -70,6 +70,8 @@ _CATALOGUE = {
     "pcg": ["csr", "vec", "vec", "scalar", "scalar"],
     "spmm": ["csr", "mat", "mat"],
     "plus_norm": ["vec", "vec"],
+    "mht": ["csr", "vec", "vec", "scalar", "scalar", "scalar"],
+    "normalize_mom2": ["vec", "vec"],
 }
 
 

@@ -66,12 +66,13 @@ __device__ __forceinline__ void st2(double *p, long long i, v2d v) { reinterpret
 __global__ __launch_bounds__(256) void cg_init_kernel(long long n, const double *__restrict__ b,
                                                       const double *__restrict__ dinv, double *__restrict__ x,
                                                       double *__restrict__ r, double *__restrict__ z,
-                                                      double *__restrict__ p, double *__restrict__ partials) {
+                                                      double *__restrict__ p, double *__restrict__ partials,
+                                                      int divide) {
   __shared__ double lds4[4];
   double rr = 0.0, rz = 0.0;
   CG_GRID_STRIDE(i, 0, n) {
     const double ri = b[i];
-    const double zi = dinv ? ri * dinv[i] : ri;
+    const double zi = dinv ? (divide ? ri / dinv[i] : ri * dinv[i]) : ri;
     r[i] = ri;
     if (dinv) z[i] = zi;
     p[i] = zi;
@@ -143,7 +144,8 @@ __global__ __launch_bounds__(256) void cg_update_xr_kernel(long long n, const do
 // z = r * dinv ; block partials of r.z     (preconditioned runs only)
 __global__ __launch_bounds__(256) void cg_precond_kernel(long long n, const double *__restrict__ r,
                                                          const double *__restrict__ dinv, double *__restrict__ z,
-                                                         const CgState *st, double *__restrict__ partials, int vec) {
+                                                         const CgState *st, double *__restrict__ partials, int vec,
+                                                         int divide) {
   __shared__ double lds4[4];
   if (st->done) return;
   double acc = 0.0;
@@ -151,20 +153,42 @@ __global__ __launch_bounds__(256) void cg_precond_kernel(long long n, const doub
   CG_GRID_STRIDE(i, 0, nv) {
     const v2d rv = ld2(r, i), dv = ld2(dinv, i);
     v2d zv;
-    zv.x = rv.x * dv.x;
-    zv.y = rv.y * dv.y;
+    zv.x = divide ? rv.x / dv.x : rv.x * dv.x;
+    zv.y = divide ? rv.y / dv.y : rv.y * dv.y;
     st2(z, i, zv);
     acc = acc + rv.x * zv.x;
     acc = acc + rv.y * zv.y;
   }
   CG_GRID_STRIDE(i, 2 * nv, n) {
     const double ri = r[i];
-    const double zi = ri * dinv[i];
+    const double zi = divide ? ri / dinv[i] : ri * dinv[i];
     z[i] = zi;
     acc = acc + ri * zi;
   }
   const double bsum = block_sum_256d(acc, lds4);
   if (threadIdx.x == 0) partials[blockIdx.x] = bsum;
+}
+
+// Elementwise pieces of the masked operator and of the moment right-hand sides
+// (examples/hitting_times.py:73-93, :166-177, :181-198).
+// mode 0: out = (d*t - out) * m     (end of plpt; t = mask*x, out holds A t)
+// mode 1: out = (d*t + out) * m     (right-hand side of the second moment; t = mom1, out holds A mom1)
+__global__ __launch_bounds__(256) void masked_combine_kernel(long long n, int mode, const double *__restrict__ d,
+                                                             const double *__restrict__ t,
+                                                             const double *__restrict__ m, double *out) {
+  CG_GRID_STRIDE(i, 0, n) {
+    const double t1 = d[i] * t[i];
+    const double t2 = mode == 0 ? t1 - out[i] : t1 + out[i];
+    out[i] = t2 * m[i];
+  }
+}
+
+__global__ __launch_bounds__(256) void normalize_mom2_kernel(long long n, const double *__restrict__ m1,
+                                                             const double *__restrict__ m2, double *__restrict__ out) {
+  CG_GRID_STRIDE(i, 0, n) {
+    const double sq = m1[i] * m1[i];
+    out[i] = sqrt(m2[i] - sq);
+  }
 }
 
 // p = z + beta p with beta = rz_next/rz.
@@ -235,10 +259,15 @@ __global__ __launch_bounds__(256) void cg_scalar_kernel(int stage, int count, co
 
 using namespace lapis;
 
-extern "C" int lapis_hip_pcg_f64_i32(lapis_hip_csr_plan *plan, int64_t n, const int32_t *pos, const int32_t *crd,
-                                     const double *val, const double *b, const double *dinv, double tol,
-                                     uint64_t maxiter, double *x, uint64_t *iters, double *relres, double *work,
-                                     lapis_hip_stream_t stream) {
+namespace {
+
+// What the solver applies as A and as the preconditioner.
+//   mask == nullptr: A p is the SpMV, z = r * prec (prec may be null: z = r)      examples/pcg_solve.py:52-101
+//   mask != nullptr: A p is plpt, y = mask*(d*(mask*p) - A (mask*p)), z = r / d   examples/hitting_times.py:97-149
+// work holds 4 vectors (5 with a mask), `stride` apart.
+int pcg_run(lapis_hip_csr_plan *plan, int64_t n, const int32_t *pos, const int32_t *crd, const double *val,
+            const double *b, const double *dinv, const double *mask, double tol, uint64_t maxiter, double *x,
+            uint64_t *iters, double *relres, double *work, lapis_hip_stream_t stream) {
   LAPIS_CHECK_INIT();
   LAPIS_REQUIRE(n >= 0, "pcg: negative size");
   LAPIS_REQUIRE(iters && relres, "pcg: null iters/relres output");
@@ -293,10 +322,12 @@ extern "C" int lapis_hip_pcg_f64_i32(lapis_hip_csr_plan *plan, int64_t n, const 
   if (!work) {
     // own scratch: an even stride keeps all four vectors 16-byte aligned
     stride = (n + 1) & ~(int64_t)1;
-    PCG_TRY(hipMalloc(&own_work, sizeof(double) * 4 * (size_t)stride));
+    PCG_TRY(hipMalloc(&own_work, sizeof(double) * (mask ? 5 : 4) * (size_t)stride));
     work = own_work;
   }
   double *r = work, *z = dinv ? work + stride : work, *p = work + 2 * stride, *Ap = work + 3 * stride;
+  double *tmp = mask ? work + 4 * stride : nullptr;
+  const int divide = mask ? 1 : 0;
   PCG_TRY(hipMalloc(&state, sizeof(CgState)));
   PCG_TRY(hipMalloc(&partials, sizeof(double) * 2 * kDotMaxBlocks));
   CgState h{};
@@ -310,7 +341,8 @@ extern "C" int lapis_hip_pcg_f64_i32(lapis_hip_csr_plan *plan, int64_t n, const 
                    (!dinv || aligned16(dinv)))
                       ? 1
                       : 0;
-  hipLaunchKernelGGL(cg_init_kernel, dim3(grid), dim3(256), 0, st, (long long)n, b, dinv, x, r, z, p, partials);
+  hipLaunchKernelGGL(cg_init_kernel, dim3(grid), dim3(256), 0, st, (long long)n, b, dinv, x, r, z, p, partials,
+                     divide);
   hipLaunchKernelGGL(cg_scalar_kernel, dim3(1), dim3(256), 0, st, (int)kStageInit, grid, partials, state, pre);
   PCG_TRY(hipGetLastError());
 
@@ -333,8 +365,15 @@ extern "C" int lapis_hip_pcg_f64_i32(lapis_hip_csr_plan *plan, int64_t n, const 
                        (unsigned long long)launched);
     }
     for (int it = 0; it < todo; ++it) {
-      // Ap = A p: the reference zero-fills Ap and accumulates (examples/pcg_solve.py:12-19)
-      PCG_RC(spmv_overwrite_f64(plan, n, n, pos, crd, val, p, Ap, stream));
+      if (mask) {
+        // plpt: tmp = mask*p ; Ap = A tmp ; Ap = (d*tmp - Ap)*mask
+        PCG_RC(lapis_hip_mult_f64(n, p, mask, tmp, stream));
+        PCG_RC(spmv_overwrite_f64(plan, n, n, pos, crd, val, tmp, Ap, stream));
+        hipLaunchKernelGGL(masked_combine_kernel, dim3(grid), dim3(256), 0, st, (long long)n, 0, dinv, tmp, mask, Ap);
+      } else {
+        // Ap = A p: the reference zero-fills Ap and accumulates (examples/pcg_solve.py:12-19)
+        PCG_RC(spmv_overwrite_f64(plan, n, n, pos, crd, val, p, Ap, stream));
+      }
       hipLaunchKernelGGL(cg_pap_kernel, dim3(grid), dim3(256), 0, st, (long long)n, p, Ap, partials, vec);
       hipLaunchKernelGGL(cg_scalar_kernel, dim3(1), dim3(256), 0, st, (int)kStagePap, grid, partials, state, pre);
       hipLaunchKernelGGL(cg_update_xr_kernel, dim3(grid), dim3(256), 0, st, (long long)n, p, Ap, x, r, state,
@@ -343,7 +382,7 @@ extern "C" int lapis_hip_pcg_f64_i32(lapis_hip_csr_plan *plan, int64_t n, const 
                          pre);
       if (pre) {
         hipLaunchKernelGGL(cg_precond_kernel, dim3(grid), dim3(256), 0, st, (long long)n, r, dinv, z, state,
-                           partials, vec);
+                           partials, vec, divide);
         hipLaunchKernelGGL(cg_scalar_kernel, dim3(1), dim3(256), 0, st, (int)kStagePrecond, grid, partials, state,
                            pre);
       }
@@ -364,5 +403,67 @@ extern "C" int lapis_hip_pcg_f64_i32(lapis_hip_csr_plan *plan, int64_t n, const 
   cleanup();
 #undef PCG_TRY
 #undef PCG_RC
+  return LAPIS_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" int lapis_hip_pcg_f64_i32(lapis_hip_csr_plan *plan, int64_t n, const int32_t *pos, const int32_t *crd,
+                                     const double *val, const double *b, const double *dinv, double tol,
+                                     uint64_t maxiter, double *x, uint64_t *iters, double *relres, double *work,
+                                     lapis_hip_stream_t stream) {
+  return pcg_run(plan, n, pos, crd, val, b, dinv, nullptr, tol, maxiter, x, iters, relres, work, stream);
+}
+
+extern "C" int lapis_hip_pcg_masked_f64_i32(lapis_hip_csr_plan *plan, int64_t n, const int32_t *pos,
+                                            const int32_t *crd, const double *val, const double *b,
+                                            const double *mask, const double *d, double tol, uint64_t maxiter,
+                                            double *x, uint64_t *iters, double *relres, double *work,
+                                            lapis_hip_stream_t stream) {
+  LAPIS_REQUIRE(n == 0 || (mask && d), "pcg_masked: null mask or diagonal");
+  return pcg_run(plan, n, pos, crd, val, b, d, mask, tol, maxiter, x, iters, relres, work, stream);
+}
+
+extern "C" int lapis_hip_mht_f64_i32(lapis_hip_csr_plan *plan, int64_t n, int64_t nnz, const int32_t *pos,
+                                     const int32_t *crd, double *val, const double *mask, const double *d,
+                                     double alpha, double tol, uint64_t maxiter, double *mom1, double *mom2,
+                                     lapis_hip_stream_t stream) {
+  LAPIS_CHECK_INIT();
+  LAPIS_REQUIRE(n >= 0 && nnz >= 0, "mht: negative size");
+  if (n == 0) return LAPIS_HIP_OK;
+  LAPIS_REQUIRE(pos && mask && d && mom1 && mom2 && (nnz == 0 || (crd && val)), "mht: null argument");
+  hipStream_t st = as_stream(stream);
+  double *bbuf = nullptr;
+  LAPIS_HIP_TRY(hipMalloc(&bbuf, sizeof(double) * (size_t)n));
+  uint64_t its = 0;
+  double res = 0.0;
+  int rc = lapis_hip_scale_f64(nnz, alpha, val, stream);  // scale_csr, in place
+  if (rc == LAPIS_HIP_OK) rc = lapis_hip_mult_f64(n, d, mask, bbuf, stream);
+  if (rc == LAPIS_HIP_OK)
+    rc = lapis_hip_pcg_masked_f64_i32(plan, n, pos, crd, val, bbuf, mask, d, tol, maxiter, mom1, &its, &res, nullptr,
+                                      stream);
+  if (rc == LAPIS_HIP_OK) rc = spmv_overwrite_f64(plan, n, n, pos, crd, val, mom1, bbuf, stream);
+  if (rc == LAPIS_HIP_OK) {
+    hipLaunchKernelGGL(masked_combine_kernel, dim3(dot_grid(n)), dim3(256), 0, st, (long long)n, 1, d,
+                       (const double *)mom1, mask, bbuf);
+    if (hipGetLastError() != hipSuccess) rc = set_error(LAPIS_HIP_ERR_RUNTIME, "mht: kernel launch failed");
+  }
+  if (rc == LAPIS_HIP_OK)
+    rc = lapis_hip_pcg_masked_f64_i32(plan, n, pos, crd, val, bbuf, mask, d, tol, maxiter, mom2, &its, &res, nullptr,
+                                      stream);
+  (void)hipStreamSynchronize(st);
+  (void)hipFree(bbuf);
+  return rc;
+}
+
+extern "C" int lapis_hip_normalize_mom2_f64(int64_t n, const double *mom1, const double *mom2, double *out,
+                                            lapis_hip_stream_t stream) {
+  LAPIS_CHECK_INIT();
+  LAPIS_REQUIRE(n >= 0, "normalize_mom2: negative size");
+  if (n == 0) return LAPIS_HIP_OK;
+  LAPIS_REQUIRE(mom1 && mom2 && out, "normalize_mom2: null argument");
+  hipLaunchKernelGGL(normalize_mom2_kernel, dim3(dot_grid(n)), dim3(256), 0, as_stream(stream), (long long)n, mom1,
+                     mom2, out);
+  LAPIS_LAUNCH_CHECK();
   return LAPIS_HIP_OK;
 }

@@ -301,3 +301,50 @@ extern "C" void py_plus_norm(lapis_memref_1d_f64 **ret0, double *ret1, lapis_mem
   set_result_1d(ret0, hout, n);
   *ret1 = sqrt(sum);
 }
+
+extern "C" void py_mht(lapis_memref_1d_f64 **ret0, lapis_memref_1d_f64 **ret1, lapis_memref_1d_i32 *pos,
+                       lapis_memref_1d_i32 *crd, lapis_memref_1d_f64 *val, const lapis_csr_specifier *spec,
+                       lapis_memref_1d_f64 *mask, lapis_memref_1d_f64 *d, double alpha, double tol, size_t maxiter) {
+  int32_t *hpos = host_data(pos, 1, "positions");
+  int32_t *hcrd = host_data(crd, 1, "coordinates");
+  double *hval = host_data(val, 1, "values");
+  double *hmask = host_data(mask, 1, "mask");
+  double *hd = host_data(d, 1, "d");
+  const CsrArgs a = csr_args(pos, crd, val->sizes[0], spec);
+  const int64_t n = d->sizes[0];  // %n = tensor.dim %d (examples/hitting_times.py:157)
+  if (a.nrows != n || a.ncols != n || mask->sizes[0] < n) module_abort("mht: A must be n x n and mask of length n");
+  double *h1 = static_cast<double *>(keep_alive_alloc(sizeof(double) * (size_t)n));
+  double *h2 = static_cast<double *>(keep_alive_alloc(sizeof(double) * (size_t)n));
+  {
+    DeviceMirror<int32_t> dpos(hpos, (size_t)n + 1), dcrd(hcrd, (size_t)a.nnz);
+    DeviceMirror<double> dval(hval, (size_t)a.nnz), dmask(hmask, (size_t)n), dd(hd, (size_t)n);
+    DeviceMirror<double> d1(h1, (size_t)n, false), d2(h2, (size_t)n, false);
+    lapis_hip_csr_plan *plan = nullptr;
+    check(lapis_hip_csr_plan_create(&plan, n, n, a.nnz, dpos.dev, dcrd.dev, 8, nullptr), "lapis_hip_csr_plan_create");
+    check(lapis_hip_mht_f64_i32(plan, n, a.nnz, dpos.dev, dcrd.dev, dval.dev, dmask.dev, dd.dev, alpha, tol,
+                                (uint64_t)maxiter, d1.dev, d2.dev, nullptr),
+          "lapis_hip_mht_f64_i32");
+    lapis_hip_csr_plan_destroy(plan);
+    d1.sync_host();
+    d2.sync_host();
+    // the scaled values stay on the device: they are no result of the function, and a
+    // DualView built from host memory is not copied back unless it is one
+  }
+  set_result_1d(ret0, h1, n);
+  set_result_1d(ret1, h2, n);
+}
+
+extern "C" void py_normalize_mom2(lapis_memref_1d_f64 **ret0, lapis_memref_1d_f64 *mom1, lapis_memref_1d_f64 *mom2) {
+  double *h1 = host_data(mom1, 1, "mom1");
+  double *h2 = host_data(mom2, 1, "mom2");
+  const int64_t n = mom1->sizes[0];
+  if (mom2->sizes[0] < n) module_abort("normalize_mom2: mom2 shorter than mom1");
+  double *hout = static_cast<double *>(keep_alive_alloc(sizeof(double) * (size_t)n));
+  {
+    DeviceMirror<double> d1(h1, (size_t)n), d2(h2, (size_t)n), dout(hout, (size_t)n, false);
+    check(lapis_hip_normalize_mom2_f64(n, d1.dev, d2.dev, dout.dev, nullptr), "lapis_hip_normalize_mom2_f64");
+    check(lapis_hip_stream_synchronize(nullptr), "stream synchronize");
+    dout.sync_host();
+  }
+  set_result_1d(ret0, hout, n);
+}

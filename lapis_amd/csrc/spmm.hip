@@ -108,6 +108,30 @@ __global__ __launch_bounds__(256) void spmm_wave_row_generic_kernel(int nrows, i
   }
 }
 
+// Batched CSRV product of examples/bspmm.py:22-50: A is CSR over (n1, n2) and every
+// non-zero carries nh values (a trailing dense batch); out(i, d, h) += A(i, c, h) * V(c, d, h).
+// One wavefront per row; lanes walk the dh*nh values of an output row, so the read of
+// a V row is coalesced and the nh batch values of a non-zero are read contiguously.
+__global__ __launch_bounds__(256) void bspmm_csrv_kernel(int n1, int dh, int nh, const int *__restrict__ pos,
+                                                         const int *__restrict__ crd,
+                                                         const float *__restrict__ val,
+                                                         const float *__restrict__ V, float *__restrict__ out) {
+  const int lane = threadIdx.x & 63;
+  const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= n1) return;
+  const int start = pos[row], end = pos[row + 1];
+  const long long K = (long long)dh * nh;
+  for (long long j = lane; j < K; j += 64) {
+    const int h = (int)(j % nh);
+    float acc = out[row * K + j];
+    for (int e = start; e < end; ++e) {
+      const float prod = val[(long long)e * nh + h] * V[(long long)crd[e] * K + j];
+      acc = prod + acc;
+    }
+    out[row * K + j] = acc;
+  }
+}
+
 template <typename T, int LPR>
 void launch_wave_row(int64_t nrows, const int *pos, const int *crd, const T *val, const T *B, int64_t ldb, T *C,
                      int64_t ldc, hipStream_t st) {
@@ -159,4 +183,21 @@ extern "C" int lapis_hip_spmm_csr_f64_i32(int64_t nrows, int64_t ncols, int64_t 
                                           const int32_t *crd, const double *val, const double *B, int64_t ldb,
                                           double *C, int64_t ldc, lapis_hip_stream_t stream) {
   return spmm_impl<double>("spmm_csr_f64", nrows, ncols, k, pos, crd, val, B, ldb, C, ldc, stream);
+}
+
+extern "C" int lapis_hip_bspmm_csrv_f32_i32(int64_t n1, int64_t n2, int64_t dh, int64_t nh, const int32_t *pos,
+                                            const int32_t *crd, const float *val, const float *V, float *out,
+                                            lapis_hip_stream_t stream) {
+  LAPIS_CHECK_INIT();
+  LAPIS_REQUIRE(n1 >= 0 && n2 >= 0 && dh >= 0 && nh >= 0, "bspmm_csrv: negative dimension");
+  LAPIS_REQUIRE(n1 <= INT32_MAX - 64 && n2 <= INT32_MAX && dh <= INT32_MAX && nh <= INT32_MAX,
+                "bspmm_csrv: dimension exceeds int32");
+  if (n1 == 0 || dh == 0 || nh == 0) return LAPIS_HIP_OK;
+  LAPIS_REQUIRE(pos && out, "bspmm_csrv: null positions or output");
+  LAPIS_REQUIRE(n2 == 0 || (crd && val && V), "bspmm_csrv: null coordinates, values or V");
+  if (n2 == 0) return LAPIS_HIP_OK;
+  hipLaunchKernelGGL(bspmm_csrv_kernel, dim3((unsigned)ceil_div(n1, 4)), dim3(256), 0, as_stream(stream), (int)n1,
+                     (int)dh, (int)nh, pos, crd, val, V, out);
+  LAPIS_LAUNCH_CHECK();
+  return LAPIS_HIP_OK;
 }

@@ -56,6 +56,7 @@ _SIGNATURES = {
     "lapis_hip_spmv_csr_f32_i32": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp],
     "lapis_hip_spmm_csr_f32_i32": [_i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp],
     "lapis_hip_spmm_csr_f64_i32": [_i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp],
+    "lapis_hip_bspmm_csrv_f32_i32": [_i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp],
     "lapis_hip_dot_f64": [_i64, _vp, _vp, _dbl, _vp, _vp],
     "lapis_hip_dot_f32": [_i64, _vp, _vp, _flt, _vp, _vp],
     "lapis_hip_axpby_f64": [_i64, _dbl, _vp, _dbl, _vp, _vp, _vp],
@@ -66,6 +67,10 @@ _SIGNATURES = {
     "lapis_hip_fill_f32": [_i64, _flt, _vp, _vp],
     "lapis_hip_copy_f64": [_i64, _vp, _vp, _vp],
     "lapis_hip_scale_f64": [_i64, _dbl, _vp, _vp],
+    "lapis_hip_pcg_masked_f64_i32": [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _dbl, _u64, _vp,
+                                     ctypes.POINTER(_u64), ctypes.POINTER(_dbl), _vp, _vp],
+    "lapis_hip_mht_f64_i32": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _dbl, _dbl, _u64, _vp, _vp, _vp],
+    "lapis_hip_normalize_mom2_f64": [_i64, _vp, _vp, _vp, _vp],
     "lapis_hip_pcg_f64_i32": [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _dbl, _u64, _vp,
                               ctypes.POINTER(_u64), ctypes.POINTER(_dbl), _vp, _vp],
 }
@@ -267,3 +272,34 @@ def pcg(plan, n, pos, crd, val, b, dinv, tol, maxiter, x, work=None, stream=None
                                     _ptr(b), _ptr(dinv), tol, maxiter, _ptr(x), ctypes.byref(iters),
                                     ctypes.byref(relres), _ptr(work), _stream(stream)))
     return int(iters.value), relres.value
+
+
+def pcg_masked(plan, n, pos, crd, val, b, mask, d, tol, maxiter, x, work=None, stream=None):
+    """Masked CG of examples/hitting_times.py:97 on device buffers -> (iters, relres)."""
+    lib = init()
+    iters, relres = _u64(0), _dbl(0.0)
+    check(lib.lapis_hip_pcg_masked_f64_i32(plan.handle if plan is not None else None, n, _ptr(pos), _ptr(crd),
+                                           _ptr(val), _ptr(b), _ptr(mask), _ptr(d), tol, maxiter, _ptr(x),
+                                           ctypes.byref(iters), ctypes.byref(relres), _ptr(work), _stream(stream)))
+    return int(iters.value), relres.value
+
+
+def mht(plan, n, pos, crd, val, mask, d, alpha, tol, maxiter, mom1, mom2, stream=None):
+    """Hitting-time moments of examples/hitting_times.py:153; scales ``val`` in place."""
+    check(init().lapis_hip_mht_f64_i32(plan.handle if plan is not None else None, n, int(val.shape[0]), _ptr(pos),
+                                       _ptr(crd), _ptr(val), _ptr(mask), _ptr(d), alpha, tol, maxiter, _ptr(mom1),
+                                       _ptr(mom2), _stream(stream)))
+    return mom1, mom2
+
+
+def normalize_mom2(mom1, mom2, out, stream=None):
+    check(init().lapis_hip_normalize_mom2_f64(int(mom1.shape[0]), _ptr(mom1), _ptr(mom2), _ptr(out), _stream(stream)))
+    return out
+
+
+def bspmm_csrv(n1, n2, pos, crd, val, V, out, stream=None):
+    """out(n1,dh,nh) += A(n1,n2,nh) * V(n2,dh,nh) with CSRV A (examples/bspmm.py)."""
+    dh, nh = int(V.shape[1]), int(V.shape[2])
+    check(init().lapis_hip_bspmm_csrv_f32_i32(n1, n2, dh, nh, _ptr(pos), _ptr(crd), _ptr(val), _ptr(V), _ptr(out),
+                                              _stream(stream)))
+    return out

@@ -138,3 +138,36 @@ class LAPISModule:
                                     ctypes.pointer(rt.get_ranked_memref_descriptor(param0)),
                                     ctypes.pointer(rt.get_ranked_memref_descriptor(param1)))
         return (rt.ranked_memref_to_numpy(ret0[0]), ret1[0])
+
+    # func @mht(A, mask, d, alpha, tol, maxiter) -> (mom1, mom2)      (examples/hitting_times.py:153,216)
+    def mht(self, param0, param1, param2, param3, param4, param5, param6, param7, param8):
+        param0 = numpy.require(param0, dtype=numpy.int32, requirements=['C'])
+        param1 = numpy.require(param1, dtype=numpy.int32, requirements=['C'])
+        param2 = numpy.require(param2, dtype=numpy.float64, requirements=['C'])
+        param3 = _flatten_specifier(param3)
+        param4 = numpy.require(param4, dtype=numpy.float64, requirements=['C'])
+        param5 = numpy.require(param5, dtype=numpy.float64, requirements=['C'])
+        param6 = ctypes.c_double(param6)
+        param7 = ctypes.c_double(param7)
+        param8 = ctypes.c_ulong(param8)
+        ret0 = ctypes.pointer(ctypes.pointer(rt.make_nd_memref_descriptor(1, ctypes.c_double)()))
+        ret1 = ctypes.pointer(ctypes.pointer(rt.make_nd_memref_descriptor(1, ctypes.c_double)()))
+        self.libHandle.py_mht(ret0, ret1,
+                              ctypes.pointer(rt.get_ranked_memref_descriptor(param0)),
+                              ctypes.pointer(rt.get_ranked_memref_descriptor(param1)),
+                              ctypes.pointer(rt.get_ranked_memref_descriptor(param2)),
+                              param3.ctypes.data_as(ctypes.c_void_p),
+                              ctypes.pointer(rt.get_ranked_memref_descriptor(param4)),
+                              ctypes.pointer(rt.get_ranked_memref_descriptor(param5)),
+                              param6, param7, param8)
+        return (rt.ranked_memref_to_numpy(ret0[0]), rt.ranked_memref_to_numpy(ret1[0]))
+
+    # func @normalize_mom2(mom1, mom2) -> stdev      (examples/hitting_times.py:181,218)
+    def normalize_mom2(self, param0, param1):
+        param0 = numpy.require(param0, dtype=numpy.float64, requirements=['C'])
+        param1 = numpy.require(param1, dtype=numpy.float64, requirements=['C'])
+        ret0 = ctypes.pointer(ctypes.pointer(rt.make_nd_memref_descriptor(1, ctypes.c_double)()))
+        self.libHandle.py_normalize_mom2(ret0,
+                                         ctypes.pointer(rt.get_ranked_memref_descriptor(param0)),
+                                         ctypes.pointer(rt.get_ranked_memref_descriptor(param1)))
+        return (rt.ranked_memref_to_numpy(ret0[0]))

@@ -83,7 +83,8 @@ class Oracle:
         n = pos.shape[0] - 1
         out = np.empty(n, dtype=np.float64)
         name = "oracle_spmv_abs_scale_%s_i32" % ("f64" if dt == np.float64 else "f32")
-        yp = _ptr(_req(yin, dt)) if yin is not None else None
+        yin = _req(yin, dt) if yin is not None else None  # held in a local: the pointer below must stay valid
+        yp = _ptr(yin) if yin is not None else None
         getattr(self.lib, name)(_c_i64(n), _ptr(pos), _ptr(crd), _ptr(val), _ptr(x), yp, _ptr(out))
         return out
 
@@ -163,6 +164,19 @@ class Oracle:
         relres = _c_dbl(0.0)
         it = self.lib.oracle_pcg_f64_i32(_c_i64(n), _ptr(pos), _ptr(crd), _ptr(val), _ptr(b), _ptr(dinv),
                                          _c_dbl(tol), _c_u64(maxiter), _ptr(x), ctypes.byref(relres), _ptr(work))
+        return x, int(it), relres.value
+
+    def pcg_masked(self, pos, crd, val, b, mask, d, tol, maxiter):
+        """examples/hitting_times.py:97 -> (x, iters, relres)."""
+        pos, crd = _req(pos, np.int32), _req(crd, np.int32)
+        val, b = _req(val, np.float64), _req(b, np.float64)
+        mask, d = _req(mask, np.float64), _req(d, np.float64)
+        n = b.shape[0]
+        x, work = np.empty(n), np.empty(5 * n)
+        relres = _c_dbl(0.0)
+        it = self.lib.oracle_pcg_masked_f64_i32(_c_i64(n), _ptr(pos), _ptr(crd), _ptr(val), _ptr(b), _ptr(mask),
+                                                _ptr(d), _c_dbl(tol), _c_u64(maxiter), _ptr(x), ctypes.byref(relres),
+                                                _ptr(work))
         return x, int(it), relres.value
 
     def mht(self, pos, crd, val, mask, d, alpha, tol, maxiter):

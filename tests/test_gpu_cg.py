@@ -74,3 +74,39 @@ def test_convergence_stops_early_and_x_is_not_touched_afterwards(gpu, oracle):
     # a huge tolerance leaves after the first update, as the reference's loop does
     _, i1, _ = _solve(gpu, A.pos, A.crd, A.val, rhs, dinv, 1e30, 50)
     assert i1 == 1
+
+
+def test_masked_cg_and_moments_match_oracle(gpu, oracle, golden):
+    g = golden["hitting_times"]
+    pos, crd, val, shape = read_mtx_csr("mht_A.mtx")
+    n = shape[0]
+    d = read_mtx_csr("mht_D.mtx")[2]
+    mask = np.ones(n)
+    mask[3] = 0
+    dpos, dcrd, dval = dev(pos), dev(crd), dev(val)
+    plan = gpu.CsrPlan(n, n, dpos, dcrd)
+    m1 = torch.empty(n, dtype=torch.float64, device="cuda")
+    m2 = torch.empty(n, dtype=torch.float64, device="cuda")
+    gpu.mht(plan, n, dpos, dcrd, dval, dev(mask), dev(d), g["alpha"], g["tol"], g["maxiter"], m1, m2)
+    assert np.array_equal(dval.cpu().numpy(), val * g["alpha"])  # scale_csr works in place, bit for bit
+    vo = val.copy()
+    o1, o2 = oracle.mht(pos, crd, vo, mask, d, g["alpha"], g["tol"], g["maxiter"])
+    assert np.allclose(m1.cpu().numpy(), o1, rtol=1e-9, atol=1e-12)
+    assert np.allclose(m2.cpu().numpy(), o2, rtol=1e-9, atol=1e-12)
+    out = torch.empty(n, dtype=torch.float64, device="cuda")
+    gpu.normalize_mom2(m1, m2, out)
+    assert np.allclose(out.cpu().numpy(), g["mom2_gold"])
+    # a larger masked system against the oracle's masked solver
+    A, b = gen.config5(scale=(14 / 192) ** 3)
+    nn = A.nrows
+    dd = np.full(nn, 6.5)
+    mk = (np.arange(nn) % 7 != 0).astype(np.float64)
+    off = A.val.copy()
+    off[off > 0] = 0.0
+    off = -off  # adjacency part of the Laplacian: plpt applies d - A
+    x = torch.empty(nn, dtype=torch.float64, device="cuda")
+    dp, dc = dev(A.pos), dev(A.crd)
+    it, rr = gpu.pcg_masked(gpu.CsrPlan(nn, nn, dp, dc), nn, dp, dc, dev(off), dev(b * mk), dev(mk), dev(dd), 1e-9, 300, x)
+    xo, ito, _ = oracle.pcg_masked(A.pos, A.crd, off, b * mk, mk, dd, 1e-9, 300)
+    assert it == ito and it < 300
+    assert np.allclose(x.cpu().numpy(), xo, rtol=1e-8, atol=1e-11)

@@ -73,6 +73,21 @@ def test_pcg_solve_example(module_kokkos, golden, oracle):
     assert int(numiter) == io and numiter.dtype == np.uint64
 
 
+def test_hitting_times_example_gold_vectors(module_kokkos, golden):
+    g = golden["hitting_times"]
+    pos, crd, val, shape = read_mtx_csr("mht_A.mtx")
+    A = sp.csr_matrix((val, crd, pos), shape=shape)
+    n, nnz = A.shape[0], A.nnz
+    D = read_mtx_csr("mht_D.mtx")[2]
+    mask = np.ones(n)
+    for s_ in g["seedset"]:
+        mask[s_] = 0
+    (mom1, mom2) = module_kokkos.mht(A.indptr, A.indices, A.data, ((n, n), (n + 1, nnz, nnz)), mask, D, g["alpha"],
+                                     g["tol"], g["maxiter"])
+    mom2_norm = module_kokkos.normalize_mom2(mom1, mom2)
+    assert np.allclose(mom1, g["mom1_gold"]) and np.allclose(mom2_norm, g["mom2_gold"])  # the reference's check
+
+
 def test_multiple_results_example(module_kokkos, golden):
     g = golden["multiple_results"]
     x, y = np.array(g["x"]), np.array(g["y"])

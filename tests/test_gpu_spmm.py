@@ -67,3 +67,26 @@ def test_spmm_strided_leading_dimensions(gpu, oracle):
     got = Cd.cpu().numpy()
     assert np.allclose(got[:, :k], want, rtol=1e-5, atol=1e-5)
     assert np.array_equal(got[:, k:], Cfull[:, k:])  # columns beyond k are untouched
+
+
+def test_batched_csrv_product_of_the_bspmm_example(gpu, oracle):
+    # the shapes and sparsity of examples/bspmm.py:62-75 with a fixed seed, then a larger case
+    for (m, n, b, k, pos, crd, seed) in [
+            (5, 6, 8, 3, np.array([0, 1, 5, 6, 8, 8], np.int32), np.array([1, 0, 2, 3, 4, 5, 0, 1], np.int32), 12),
+            (None, None, 5, 7, None, None, 13)]:
+        rng = np.random.default_rng(seed)
+        if m is None:
+            A = gen.fixed_degree_random(300, 9, seed=41)
+            m = n = 300
+            pos, crd = A.pos, A.crd
+        nnz = crd.shape[0]
+        values = rng.uniform(1.0, 2.0, nnz * b).astype(np.float32)
+        V = rng.uniform(1.0, 2.0, (n, k, b)).astype(np.float32)
+        gold = np.zeros((m, k, b), np.float32)
+        for i in range(b):
+            gold[:, :, i] = sp.csr_matrix((values[i::b], crd, pos), (m, n)) @ V[:, :, i]
+        out = torch.zeros(m, k, b, dtype=torch.float32, device="cuda")
+        gpu.bspmm_csrv(m, n, dev(pos), dev(crd), dev(values), dev(V), out)
+        torch.cuda.synchronize()
+        assert np.allclose(gold, out.cpu().numpy())  # the example's acceptance check
+        assert np.array_equal(out.cpu().numpy(), oracle.bspmm_csrv(pos, crd, values, V, m))  # same order: bit-exact
