@@ -95,7 +95,7 @@ typedef struct lapis_hip_csr_stats {
   /* what this plan launches */
   int32_t kernel;      /* enum lapis_hip_spmv_kernel, never AUTO */
   int32_t width;       /* lanes per row for SUBWARP, else 0 */
-  int32_t chunk;       /* non-zeros per wavefront for NNZSPLIT, else 0 */
+  int32_t chunk;       /* non-zeros per wavefront for NNZSPLIT (512, 1024 or 2048), else 0 */
   /* 1 if lapis_hip_csr_plan_build_colblock is expected to pay for this matrix (x far
    * larger than an XCD's L2, gathers spread all over it, even rows); plan creation
    * cannot build it itself because it is not given the values */

@@ -10,6 +10,8 @@ struct lapis_hip_csr_plan {
   lapis_hip_csr_stats stats;
   const int32_t *pos;
   int nchunks;
+  int chunk;            // non-zeros per wavefront of the row-split kernel (512, 1024 or 2048)
+  int waves_per_block;  // wavefronts per workgroup of the row-split kernel
   bool nontemporal;
   // row-split (NNZSPLIT) metadata
   int *chunk_row;    // device, int[nchunks+1]

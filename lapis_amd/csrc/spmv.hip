@@ -430,7 +430,7 @@ void choose_kernel(lapis_hip_csr_plan *p) {
   }
   if (skewed || mean < 2048.0) {
     s.kernel = LAPIS_HIP_SPMV_NNZSPLIT;
-    s.chunk = kChunk;
+    s.chunk = p->chunk;
     return;
   }
   // very long, even rows: a whole wavefront per row
@@ -478,23 +478,40 @@ int launch_rowblock(int64_t nrows, int64_t nnz, const int *pos, const int *crd, 
   return LAPIS_HIP_OK;
 }
 
-template <typename T, bool VEC, bool NT>
-int launch_nnzsplit(const lapis_hip_csr_plan *p, const int *pos, const int *crd, const T *val, const T *x,
-                    T *y, hipStream_t st, int accumulate = 1) {
+template <typename T, bool VEC, bool NT, int CH, int WPB>
+int launch_nnzsplit_cfg(const lapis_hip_csr_plan *p, const int *pos, const int *crd, const T *val, const T *x,
+                        T *y, hipStream_t st, int accumulate) {
   const int nchunks = p->nchunks;
-  const int blocks = (int)ceil_div(nchunks, kWavesPerBlock);
-  launch_timed(spmv_nnzsplit_kernel<T, kChunk, kWavesPerBlock, VEC, NT>, dim3(blocks), dim3(64 * kWavesPerBlock),
+  const int blocks = (int)ceil_div(nchunks, WPB);
+  launch_timed(spmv_nnzsplit_kernel<T, CH, WPB, VEC, NT>, dim3(blocks), dim3(64 * WPB),
                st, (int)p->stats.nrows, (int)p->stats.nnz, nchunks, pos, crd, val, x, y,
                (const int *)p->chunk_row, static_cast<T *>(p->part_first), static_cast<T *>(p->part_last), accumulate);
   LAPIS_LAUNCH_CHECK();
   if (nchunks > 1) {
     const int fblocks = (int)ceil_div(nchunks - 1, 256);
-    hipLaunchKernelGGL((spmv_nnzsplit_fixup_kernel<T, kChunk>), dim3(fblocks), dim3(256), 0, st, nchunks, pos,
+    hipLaunchKernelGGL((spmv_nnzsplit_fixup_kernel<T, CH>), dim3(fblocks), dim3(256), 0, st, nchunks, pos,
                        p->chunk_row, static_cast<const T *>(p->part_first),
                        static_cast<const T *>(p->part_last), y, accumulate);
     LAPIS_LAUNCH_CHECK();
   }
   return LAPIS_HIP_OK;
+}
+
+template <typename T, bool VEC, bool NT>
+int launch_nnzsplit(const lapis_hip_csr_plan *p, const int *pos, const int *crd, const T *val, const T *x,
+                    T *y, hipStream_t st, int accumulate = 1) {
+  switch (p->stats.chunk * 16 + p->waves_per_block) {
+    case 512 * 16 + 4: return launch_nnzsplit_cfg<T, VEC, NT, 512, 4>(p, pos, crd, val, x, y, st, accumulate);
+    case 512 * 16 + 8: return launch_nnzsplit_cfg<T, VEC, NT, 512, 8>(p, pos, crd, val, x, y, st, accumulate);
+    case 1024 * 16 + 2: return launch_nnzsplit_cfg<T, VEC, NT, 1024, 2>(p, pos, crd, val, x, y, st, accumulate);
+    case 1024 * 16 + 4: return launch_nnzsplit_cfg<T, VEC, NT, 1024, 4>(p, pos, crd, val, x, y, st, accumulate);
+    case 1024 * 16 + 8: return launch_nnzsplit_cfg<T, VEC, NT, 1024, 8>(p, pos, crd, val, x, y, st, accumulate);
+    case 2048 * 16 + 2: return launch_nnzsplit_cfg<T, VEC, NT, 2048, 2>(p, pos, crd, val, x, y, st, accumulate);
+    case 2048 * 16 + 4: return launch_nnzsplit_cfg<T, VEC, NT, 2048, 4>(p, pos, crd, val, x, y, st, accumulate);
+    default:
+      return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT, "spmv: no row-split kernel for %d non-zeros per wavefront, %d wavefronts per block",
+                       p->stats.chunk, p->waves_per_block);
+  }
 }
 
 template <typename T>
@@ -671,7 +688,15 @@ extern "C" int lapis_hip_csr_plan_create(lapis_hip_csr_plan **out, int64_t nrows
   // keep the stream from evicting what little of x is cached); when the gathers of a
   // chunk stay inside a window L2 can hold, plain loads are 10-15 % faster.
   p->nontemporal = env_int("LAPIS_HIP_SPMV_NONTEMPORAL", s.mean_chunk_col_span * value_bytes > 2.0 * 1024 * 1024) != 0;
-  p->nchunks = (int)ceil_div(nnz, kChunk);
+  // Measured: 512 non-zeros per wavefront in workgroups of 8 for short rows (7-point
+  // stencil: +4 to +8 % over 1024 x 4), 1024 in workgroups of 2 from about 32 per row on.
+  p->chunk = env_int("LAPIS_HIP_SPMV_CHUNK", s.mean_row_len < 32.0 ? 512 : 1024);
+  if (p->chunk != 512 && p->chunk != 2048) p->chunk = 1024;
+  p->waves_per_block = env_int("LAPIS_HIP_SPMV_WAVES", p->chunk == 512 ? 8 : 2);
+  if (p->waves_per_block != 2 && p->waves_per_block != 4 && p->waves_per_block != 8) p->waves_per_block = 4;
+  if (p->chunk == 2048 && p->waves_per_block == 8) p->waves_per_block = 4;
+  if (p->chunk == 512 && p->waves_per_block == 2) p->waves_per_block = 4;
+  p->nchunks = (int)ceil_div(nnz, p->chunk);
   choose_kernel(p);
 
   // Row-split metadata is built whatever the choice, so that set_kernel can switch to it.
@@ -680,8 +705,13 @@ extern "C" int lapis_hip_csr_plan_create(lapis_hip_csr_plan **out, int64_t nrows
     if (e == hipSuccess) e = hipMalloc(&p->part_first, 8 * (size_t)p->nchunks);
     if (e == hipSuccess) e = hipMalloc(&p->part_last, 8 * (size_t)p->nchunks);
     if (e == hipSuccess) {
-      hipLaunchKernelGGL((chunk_row_kernel<kChunk>), dim3((unsigned)ceil_div(nrows, 256)), dim3(256), 0, st,
-                         (int)nrows, p->nchunks, pos, p->chunk_row);
+      const dim3 g((unsigned)ceil_div(nrows, 256));
+      if (p->chunk == 512)
+        hipLaunchKernelGGL((chunk_row_kernel<512>), g, dim3(256), 0, st, (int)nrows, p->nchunks, pos, p->chunk_row);
+      else if (p->chunk == 2048)
+        hipLaunchKernelGGL((chunk_row_kernel<2048>), g, dim3(256), 0, st, (int)nrows, p->nchunks, pos, p->chunk_row);
+      else
+        hipLaunchKernelGGL((chunk_row_kernel<1024>), g, dim3(256), 0, st, (int)nrows, p->nchunks, pos, p->chunk_row);
       e = hipGetLastError();
     }
     if (e == hipSuccess) e = hipStreamSynchronize(st);
@@ -720,7 +750,7 @@ extern "C" int lapis_hip_csr_plan_set_kernel(lapis_hip_csr_plan *plan, int kerne
     case LAPIS_HIP_SPMV_NNZSPLIT:
       s.kernel = kernel;
       s.width = 0;
-      s.chunk = kChunk;
+      s.chunk = plan->chunk;
       return LAPIS_HIP_OK;
     case LAPIS_HIP_SPMV_COLBLOCK:
       if (!plan->colblock_built)

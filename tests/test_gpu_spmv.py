@@ -75,6 +75,24 @@ def test_spmv_matches_oracle(gpu, cases, kernel, width):
         plan.destroy()
 
 
+@pytest.mark.parametrize("chunk,waves", [(512, 4), (512, 8), (1024, 2), (1024, 4), (1024, 8), (2048, 2), (2048, 4)])
+def test_row_split_kernel_at_every_chunk_size(gpu, cases, monkeypatch, chunk, waves):
+    dtype, built = cases
+    monkeypatch.setenv("LAPIS_HIP_SPMV_CHUNK", str(chunk))
+    monkeypatch.setenv("LAPIS_HIP_SPMV_WAVES", str(waves))
+    for name, (A, x, y_in, want, scale) in built.items():
+        print("case", name, "nnzsplit", chunk, waves, np.dtype(dtype).name, flush=True)
+        pos, crd, val = dev(A.pos), dev(A.crd), dev(A.val)
+        plan = gpu.CsrPlan(A.nrows, A.ncols, pos, crd, value_bytes=np.dtype(dtype).itemsize).set_kernel(3)
+        if A.nnz:
+            assert plan.stats()["chunk"] == chunk
+        y = dev(y_in)
+        gpu.spmv(plan, A.nrows, A.ncols, pos, crd, val, dev(x), y)
+        torch.cuda.synchronize()
+        assert_rows_close(y.cpu().numpy(), want, scale, dtype, "%s/nnzsplit%dx%d" % (name, chunk, waves))
+        plan.destroy()
+
+
 @pytest.mark.parametrize("slice_log2", [0, 4, 9])
 def test_column_blocked_copy_matches_oracle(gpu, cases, slice_log2):
     dtype, built = cases
