@@ -176,7 +176,8 @@ __global__ __launch_bounds__(64 * WAVES) void spmv_colblock_kernel(int nrows, in
 }
 
 // key = (row block << (32 + slice bits)) | (slice << 32) | (row in block << col_bits) | column
-__global__ __launch_bounds__(256) void colblock_keys_kernel(int nrows, int col_bits, int slice_log2, int slice_bits,
+__global__ __launch_bounds__(256) void colblock_keys_kernel(int nrows, int rows_per_block, int col_bits,
+                                                            int slice_log2, int slice_bits,
                                                             const int *__restrict__ pos,
                                                             const int *__restrict__ crd,
                                                             unsigned long long *__restrict__ keys) {
@@ -184,8 +185,8 @@ __global__ __launch_bounds__(256) void colblock_keys_kernel(int nrows, int col_b
   const int lane = threadIdx.x & 63;
   const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= nrows) return;
-  const unsigned long long rb = (unsigned long long)(row / kColblockRows);
-  const unsigned long long rl = (unsigned long long)(row % kColblockRows);
+  const unsigned long long rb = (unsigned long long)(row / rows_per_block);
+  const unsigned long long rl = (unsigned long long)(row % rows_per_block);
   const int s = pos[row], e = pos[row + 1];
   for (int j = s + lane; j < e; j += 64) {
     const unsigned long long c = (unsigned long long)(unsigned)crd[j];
@@ -207,44 +208,42 @@ void free_colblock(lapis_hip_csr_plan *p) {
   p->colblock_built = false;
 }
 
-template <typename T, int STEPS, int EPL, int PAD>
+template <typename T, int RB, int WAVES, int STEPS, int EPL>
 int launch_colblock_cfg(const lapis_hip_csr_plan *p, const int *pos, const T *x, T *y, hipStream_t st) {
-  constexpr int WAVES = 4;
-  const int64_t nrb = ceil_div(p->stats.nrows, kColblockRows);
+  const int64_t nrb = ceil_div(p->stats.nrows, RB);
   const dim3 grid((unsigned)ceil_div(nrb, WAVES)), block(64 * WAVES);
   if (p->nontemporal)
-    launch_timed(spmv_colblock_kernel<T, kColblockRows, WAVES, STEPS, EPL, PAD, true>, grid, block, st,
-                 (int)p->stats.nrows, (int)p->stats.nnz, p->colblock_col_bits, pos,
-                 (const unsigned *)p->colblock_idx, (const T *)p->colblock_val, x, y, p->colblock_pace_fp);
+    launch_timed(spmv_colblock_kernel<T, RB, WAVES, STEPS, EPL, 0, true>, grid, block, st, (int)p->stats.nrows,
+                 (int)p->stats.nnz, p->colblock_col_bits, pos, (const unsigned *)p->colblock_idx,
+                 (const T *)p->colblock_val, x, y, p->colblock_pace_fp);
   else
-    launch_timed(spmv_colblock_kernel<T, kColblockRows, WAVES, STEPS, EPL, PAD, false>, grid, block, st,
-                 (int)p->stats.nrows, (int)p->stats.nnz, p->colblock_col_bits, pos,
-                 (const unsigned *)p->colblock_idx, (const T *)p->colblock_val, x, y, p->colblock_pace_fp);
+    launch_timed(spmv_colblock_kernel<T, RB, WAVES, STEPS, EPL, 0, false>, grid, block, st, (int)p->stats.nrows,
+                 (int)p->stats.nnz, p->colblock_col_bits, pos, (const unsigned *)p->colblock_idx,
+                 (const T *)p->colblock_val, x, y, p->colblock_pace_fp);
   LAPIS_LAUNCH_CHECK();
   return LAPIS_HIP_OK;
 }
 
-template <typename T>
-int launch_colblock(const lapis_hip_csr_plan *p, const int *pos, const T *x, T *y, hipStream_t st) {
-  constexpr int PADW = (40960 - 4 * kColblockRows * (int)sizeof(T)) / (int)sizeof(T);  // 40 KB per workgroup
-  const int key = p->colblock_steps * 100 + p->colblock_epl * 10 + (p->colblock_pad ? 1 : 0);
-  switch (key) {
-    case 140: return launch_colblock_cfg<T, 1, 4, 0>(p, pos, x, y, st);
-    case 141: return launch_colblock_cfg<T, 1, 4, PADW>(p, pos, x, y, st);
-    case 240: return launch_colblock_cfg<T, 2, 4, 0>(p, pos, x, y, st);
-    case 241: return launch_colblock_cfg<T, 2, 4, PADW>(p, pos, x, y, st);
-    case 120: return launch_colblock_cfg<T, 1, 2, 0>(p, pos, x, y, st);
-    case 121: return launch_colblock_cfg<T, 1, 2, PADW>(p, pos, x, y, st);
-    case 220: return launch_colblock_cfg<T, 2, 2, 0>(p, pos, x, y, st);
-    case 221: return launch_colblock_cfg<T, 2, 2, PADW>(p, pos, x, y, st);
-    case 110: return launch_colblock_cfg<T, 1, 1, 0>(p, pos, x, y, st);
-    case 111: return launch_colblock_cfg<T, 1, 1, PADW>(p, pos, x, y, st);
-    case 210: return launch_colblock_cfg<T, 2, 1, 0>(p, pos, x, y, st);
-    case 211: return launch_colblock_cfg<T, 2, 1, PADW>(p, pos, x, y, st);
+template <typename T, int RB, int WAVES>
+int launch_colblock_rb(const lapis_hip_csr_plan *p, const int *pos, const T *x, T *y, hipStream_t st) {
+  switch (p->colblock_steps * 10 + p->colblock_epl) {
+    case 22: return launch_colblock_cfg<T, RB, WAVES, 2, 2>(p, pos, x, y, st);
+    case 12: return launch_colblock_cfg<T, RB, WAVES, 1, 2>(p, pos, x, y, st);
+    case 24: return launch_colblock_cfg<T, RB, WAVES, 2, 4>(p, pos, x, y, st);
+    case 14: return launch_colblock_cfg<T, RB, WAVES, 1, 4>(p, pos, x, y, st);
     default:
       return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT, "colblock: no kernel for steps=%d entries-per-lane=%d",
                        p->colblock_steps, p->colblock_epl);
   }
+}
+
+template <typename T>
+int launch_colblock(const lapis_hip_csr_plan *p, const int *pos, const T *x, T *y, hipStream_t st) {
+  if (p->colblock_rows == 512)
+    return p->colblock_pad ? launch_colblock_rb<T, 512, 8>(p, pos, x, y, st)
+                           : launch_colblock_rb<T, 512, 4>(p, pos, x, y, st);
+  return p->colblock_pad ? launch_colblock_rb<T, 1024, 8>(p, pos, x, y, st)
+                         : launch_colblock_rb<T, 1024, 4>(p, pos, x, y, st);
 }
 template int launch_colblock<double>(const lapis_hip_csr_plan *, const int *, const double *, double *, hipStream_t);
 template int launch_colblock<float>(const lapis_hip_csr_plan *, const int *, const float *, float *, hipStream_t);
@@ -295,7 +294,7 @@ int calibrate_pace(lapis_hip_csr_plan *p, hipStream_t st) {
     return best;
   };
   const double free_ms = time_ms(0);
-  const double entries_per_wave = (double)p->stats.nnz / (double)ceil_div(nrows, kColblockRows);
+  const double entries_per_wave = (double)p->stats.nnz / (double)ceil_div(nrows, p->colblock_rows);
   unsigned best_pace = 0;
   int best_pct = 0;
   double best_ms = free_ms * 0.98;
@@ -330,7 +329,11 @@ template <typename T>
 int build(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int slice_log2, hipStream_t st) {
   const int64_t nnz = p->stats.nnz, nrows = p->stats.nrows;
   const int col_bits = std::max(1, bits_for(p->stats.ncols));
-  const int rb_bits = bits_for(ceil_div(nrows, kColblockRows));
+  {
+    const char *rows = getenv("LAPIS_HIP_COLBLOCK_ROWS");
+    p->colblock_rows = (rows && atoi(rows) == 512) ? 512 : 1024;
+  }
+  const int rb_bits = bits_for(ceil_div(nrows, p->colblock_rows));
   // the 64-bit sort key holds row block | slice | 32-bit entry word: slices must be
   // coarse enough for all three to fit
   slice_log2 = std::max(slice_log2, col_bits - (32 - rb_bits));
@@ -357,7 +360,8 @@ int build(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int slice_log
   if ((e = hipMalloc(&keys_out, sizeof(unsigned long long) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
   if ((e = hipMalloc(&val_out, sizeof(T) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
   if ((e = hipMalloc(&idx, sizeof(unsigned) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
-  hipLaunchKernelGGL(colblock_keys_kernel, dim3((unsigned)ceil_div(nrows, 4)), dim3(256), 0, st, (int)nrows, col_bits,
+  hipLaunchKernelGGL(colblock_keys_kernel, dim3((unsigned)ceil_div(nrows, 4)), dim3(256), 0, st, (int)nrows,
+                     p->colblock_rows, col_bits,
                      slice_log2, slice_bits, p->pos, crd, keys_in);
   if ((e = hipGetLastError()) != hipSuccess) return fail(e, "key kernel");
   if ((e = hipcub::DeviceRadixSort::SortPairs(nullptr, temp_bytes, keys_in, keys_out, val, val_out, (int)nnz, 0,

@@ -110,6 +110,17 @@ __device__ __forceinline__ T group_sum(T v) {
   return v;
 }
 
+// Workgroups are handed to the 8 XCDs round-robin (workgroup b runs on XCD b % 8), and
+// each XCD has its own L2.  With this map XCD k works on the k-th contiguous eighth
+// of the logical blocks instead of every eighth one, so neighbouring blocks, which
+// gather from overlapping parts of x, share an L2.  A bijection on [0, nblocks).
+constexpr int kXcds = 8;
+__device__ __forceinline__ unsigned xcd_contiguous_block(unsigned b, unsigned nblocks) {
+  const unsigned xcd = b % kXcds, idx = b / kXcds;
+  const unsigned q = nblocks / kXcds, r = nblocks % kXcds;
+  return xcd * q + (xcd < r ? xcd : r) + idx;
+}
+
 // Orders LDS traffic between the lanes of ONE wavefront (no s_barrier): LDS
 // operations of a wave execute in issue order, the fences stop the compiler from
 // moving accesses across this point.

@@ -13,6 +13,7 @@ struct lapis_hip_csr_plan {
   int chunk;            // non-zeros per wavefront of the row-split kernel (512, 1024 or 2048)
   int waves_per_block;  // wavefronts per workgroup of the row-split kernel
   bool nontemporal;
+  int xcd_map;          // 1: contiguous ranges of blocks per XCD (see xcd_contiguous_block)
   // row-split (NNZSPLIT) metadata
   int *chunk_row;    // device, int[nchunks+1]
   void *part_first;  // device, 8 bytes * nchunks
@@ -26,7 +27,8 @@ struct lapis_hip_csr_plan {
   void *colblock_val;        // device, T[nnz]
   int colblock_steps;        // steps per wavefront trip
   int colblock_epl;          // entries per lane per step (1, 2 or 4)
-  int colblock_pad;          // pad LDS so that exactly four workgroups fit a CU
+  int colblock_pad;          // 1: workgroups of 8 wavefronts instead of 4
+  int colblock_rows;         // rows per wavefront (512 or 1024)
   unsigned colblock_pace_fp; // clock ticks per entry (16.16 fixed point) of the time-triggered pacing, 0 = off
   double colblock_free_ms;   // calibration: kernel time without pacing
   double colblock_paced_ms;  // calibration: kernel time at the chosen pace

@@ -163,11 +163,12 @@ __global__ __launch_bounds__(256) void spmv_subwarp_kernel(int nrows, const int 
 template <typename T, int CAP, int WAVES, bool VEC, bool NT>
 __global__ __launch_bounds__(64 * WAVES) void spmv_rowblock_kernel(
     int nrows, int nnz, const int *__restrict__ pos, const int *__restrict__ crd,
-    const T *__restrict__ val, const T *__restrict__ x, T *__restrict__ y) {
+    const T *__restrict__ val, const T *__restrict__ x, T *__restrict__ y, int xcd_map) {
   __shared__ T lds[WAVES * CAP];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const long long row0 = ((long long)blockIdx.x * WAVES + wave) * 64;
+  const unsigned blk = xcd_map ? xcd_contiguous_block(blockIdx.x, gridDim.x) : blockIdx.x;
+  const long long row0 = ((long long)blk * WAVES + wave) * 64;
   if (row0 >= nrows) return;
   T *buf = lds + wave * CAP;
   const long long row = row0 + lane;
@@ -206,11 +207,13 @@ template <typename T, int CH, int WAVES, bool VEC, bool NT>
 __global__ __launch_bounds__(64 * WAVES) void spmv_nnzsplit_kernel(
     int nrows, int nnz, int nchunks, const int *__restrict__ pos, const int *__restrict__ crd,
     const T *__restrict__ val, const T *__restrict__ x, T *__restrict__ y,
-    const int *__restrict__ chunk_row, T *__restrict__ part_first, T *__restrict__ part_last, int accumulate) {
+    const int *__restrict__ chunk_row, T *__restrict__ part_first, T *__restrict__ part_last, int accumulate,
+    int xcd_map) {
   __shared__ T lds[WAVES * CH];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int c = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * WAVES + wave));
+  const unsigned blk = xcd_map ? xcd_contiguous_block(blockIdx.x, gridDim.x) : blockIdx.x;
+  const int c = __builtin_amdgcn_readfirstlane((int)(blk * WAVES + wave));
   if (c >= nchunks) return;
   T *buf = lds + wave * CH;
   const int e0 = c * CH;
@@ -470,10 +473,10 @@ int launch_subwarp(int width, int64_t nrows, const int *pos, const int *crd, con
 
 template <typename T, bool VEC, bool NT>
 int launch_rowblock(int64_t nrows, int64_t nnz, const int *pos, const int *crd, const T *val, const T *x,
-                    T *y, hipStream_t st) {
+                    T *y, hipStream_t st, int xcd_map) {
   const int64_t blocks = ceil_div(nrows, 64 * kWavesPerBlock);
   launch_timed(spmv_rowblock_kernel<T, kRowblockCap, kWavesPerBlock, VEC, NT>, dim3((unsigned)blocks),
-               dim3(64 * kWavesPerBlock), st, (int)nrows, (int)nnz, pos, crd, val, x, y);
+               dim3(64 * kWavesPerBlock), st, (int)nrows, (int)nnz, pos, crd, val, x, y, xcd_map);
   LAPIS_LAUNCH_CHECK();
   return LAPIS_HIP_OK;
 }
@@ -485,7 +488,8 @@ int launch_nnzsplit_cfg(const lapis_hip_csr_plan *p, const int *pos, const int *
   const int blocks = (int)ceil_div(nchunks, WPB);
   launch_timed(spmv_nnzsplit_kernel<T, CH, WPB, VEC, NT>, dim3(blocks), dim3(64 * WPB),
                st, (int)p->stats.nrows, (int)p->stats.nnz, nchunks, pos, crd, val, x, y,
-               (const int *)p->chunk_row, static_cast<T *>(p->part_first), static_cast<T *>(p->part_last), accumulate);
+               (const int *)p->chunk_row, static_cast<T *>(p->part_first), static_cast<T *>(p->part_last), accumulate,
+               p->xcd_map);
   LAPIS_LAUNCH_CHECK();
   if (nchunks > 1) {
     const int fblocks = (int)ceil_div(nchunks - 1, 256);
@@ -556,9 +560,9 @@ int spmv_impl(lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, const int3
                 : launch_subwarp<T, false>(s.width, nrows, pos, crd, val, x, y, st);
     case LAPIS_HIP_SPMV_ROWBLOCK:
       if (vec)
-        return nt ? launch_rowblock<T, true, true>(nrows, s.nnz, pos, crd, val, x, y, st)
-                  : launch_rowblock<T, true, false>(nrows, s.nnz, pos, crd, val, x, y, st);
-      return launch_rowblock<T, false, true>(nrows, s.nnz, pos, crd, val, x, y, st);
+        return nt ? launch_rowblock<T, true, true>(nrows, s.nnz, pos, crd, val, x, y, st, plan->xcd_map)
+                  : launch_rowblock<T, true, false>(nrows, s.nnz, pos, crd, val, x, y, st, plan->xcd_map);
+      return launch_rowblock<T, false, true>(nrows, s.nnz, pos, crd, val, x, y, st, plan->xcd_map);
     case LAPIS_HIP_SPMV_NNZSPLIT:
       if (vec)
         return nt ? launch_nnzsplit<T, true, true>(plan, pos, crd, val, x, y, st)
@@ -688,6 +692,10 @@ extern "C" int lapis_hip_csr_plan_create(lapis_hip_csr_plan **out, int64_t nrows
   // keep the stream from evicting what little of x is cached); when the gathers of a
   // chunk stay inside a window L2 can hold, plain loads are 10-15 % faster.
   p->nontemporal = env_int("LAPIS_HIP_SPMV_NONTEMPORAL", s.mean_chunk_col_span * value_bytes > 2.0 * 1024 * 1024) != 0;
+  // Contiguous block ranges per XCD measured no better than the hardware's round-robin
+  // (7-point stencil, n = 7.1M: 0.284 against 0.275 ms per CG iteration; neutral on the
+  // others), so it stays an opt-in.
+  p->xcd_map = env_int("LAPIS_HIP_SPMV_XCD_MAP", 0) != 0;
   // Measured: 512 non-zeros per wavefront in workgroups of 8 for short rows (7-point
   // stencil: +4 to +8 % over 1024 x 4), 1024 in workgroups of 2 from about 32 per row on.
   p->chunk = env_int("LAPIS_HIP_SPMV_CHUNK", s.mean_row_len < 32.0 ? 512 : 1024);
