@@ -96,7 +96,7 @@ def run_spmv(args, cfg):
     build_ms = None
     if args.kernel == "colblock" or (args.kernel is None and plan.stats()["colblock_recommended"]):
         t0 = time.perf_counter()
-        plan.build_colblock(crd, val)
+        plan.build_colblock(crd, val, layout=args.colblock_layout)
         torch.cuda.synchronize()
         build_ms = (time.perf_counter() - t0) * 1e3
     elif args.kernel:
@@ -114,7 +114,8 @@ def run_spmv(args, cfg):
     kt = hip.kernel_timing_stop()
     bytes_step = A.spmv_bytes()
     ms = elapsed / args.steps * 1e3
-    kernel_name = "spmv_%s_kernel<%s>" % (stats["kernel_name"], "double" if dtype == np.float64 else "float")
+    family = "colgroup" if stats["colblock_layout_name"] == "group" else stats["kernel_name"]
+    kernel_name = "spmv_%s_kernel<%s>" % (family, "double" if dtype == np.float64 else "float")
     achieved = bytes_step / (kt["mean_ms"] * 1e-3) / 1e9
     out = {
         "metric": "CSR SpMV %s achieved HBM GB/s" % ("fp64" if dtype == np.float64 else "fp32"),
@@ -125,13 +126,14 @@ def run_spmv(args, cfg):
         "config": {"workload": name, "nrows": A.nrows, "nnz": A.nnz, "seed": {0: 77, 1: 1001, 2: 2002, 3: 3003}[cfg],
                    "colblock_build_ms": build_ms, "mean_chunk_col_span": stats["mean_chunk_col_span"],
                    "algorithmic_bytes_per_step": bytes_step, "kernel": stats["kernel_name"],
+                   "colblock_layout": stats["colblock_layout_name"],
                    "width": stats["width"], "chunk": stats["chunk"],
                    "reference_vector_length": stats["reference_vector_length"], "plan_ms": plan_ms},
         "pct_of_hbm_peak": 100.0 * bytes_step / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "gflops": 2.0 * A.nnz / (ms * 1e-3) / 1e9,
         "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": traffic_from_profiles("%s_config%d" % (stats["kernel_name"], cfg)) if cfg else None,
+                     "traffic": traffic_from_profiles("%s_config%d" % (family, cfg)) if cfg else None,
                      "kernel_ms_mean": kt["mean_ms"], "kernel_ms_min": kt["min_ms"], "launches_timed": kt["count"]},
     }
     if published:
@@ -269,6 +271,8 @@ def main():
                     help="SpMV on the structure of one of the reference's published matrices instead of a config")
     ap.add_argument("--kernel", choices=["subwarp", "rowblock", "nnzsplit", "colblock"], default=None,
                     help="force an SpMV kernel family instead of the plan's choice")
+    ap.add_argument("--colblock-layout", choices=["auto", "wave", "group"], default="auto",
+                    help="layout of the column-blocked copy (auto = group)")
     ap.add_argument("--width", type=int, default=0, help="lanes per row with --kernel subwarp (0 = the reference's rule)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calibrate-copy", action="store_true",

@@ -100,7 +100,8 @@ typedef struct lapis_hip_csr_stats {
    * larger than an XCD's L2, gathers spread all over it, even rows); plan creation
    * cannot build it itself because it is not given the values */
   int32_t colblock_recommended;
-  int32_t reserved;
+  /* enum lapis_hip_colblock_layout of the copy this plan holds, 0 if none */
+  int32_t colblock_layout;
 } lapis_hip_csr_stats;
 
 typedef struct lapis_hip_csr_plan lapis_hip_csr_plan;
@@ -120,18 +121,34 @@ int lapis_hip_csr_plan_create(lapis_hip_csr_plan **plan, int64_t nrows, int64_t 
  * (0 = the reference's rule); other kernels ignore it. */
 int lapis_hip_csr_plan_set_kernel(lapis_hip_csr_plan *plan, int kernel, int width);
 int lapis_hip_csr_plan_get_stats(const lapis_hip_csr_plan *plan, lapis_hip_csr_stats *stats);
-/* Opt-in layout for matrices whose x does not fit the 4 MB L2 of an XCD (wide,
- * uniformly random columns): copies crd/val once into an order in which each
- * wavefront owns 1024 consecutive rows and walks their non-zeros slice by slice of
- * x (2^slice_log2_cols columns per slice, 0 = 1 MB of x), so that the whole chip
- * gathers from the same few slices at a time and they stay in L2.  Same 4+sizeof(T)
- * bytes per non-zero as CSR.  The reference has no counterpart (its launch never
- * looks at columns, KokkosLoopMapping.cpp:861-862).  Needs
- * ceil(log2(ncols)) <= 22.  The copy holds the VALUES as they are now: build again
- * after changing val.  Selects the COLBLOCK kernel on success; SpMV calls with this
- * plan then ignore their crd/val arguments.  Synchronises `stream`. */
+/* Opt-in layouts for matrices whose x does not fit the 4 MB L2 of an XCD (wide,
+ * uniformly random columns).  crd/val are copied once into an order in which a
+ * block of consecutive rows walks its non-zeros slice by slice of x
+ * (2^slice_log2_cols columns per slice, 0 = default), with the row sums of the block
+ * in LDS; all blocks are resident and walk the slices together, so the chip gathers
+ * from the same few slices at a time and they stay in L2.  Same 4+sizeof(T) bytes
+ * per non-zero as CSR.
+ *   WAVE : one wavefront per 1024 rows, entries of a tile in row order, the
+ *          wavefronts paced by the clock (pace calibrated here, a few launches).
+ *          Sums are added in a fixed order: results repeat bit for bit.  Needs
+ *          ceil(log2(ncols)) <= 22.
+ *   GROUP: one workgroup per up to 16384 rows, entries of a tile in COLUMN order,
+ *          so neighbouring lanes gather from the same 128-byte lines (fewer requests
+ *          to L2, which is what bounds these matrices).  Row sums are LDS atomics
+ *          shared by the wavefronts of the group: the order of additions, and with it
+ *          the last bits of y, can differ between runs.  AUTO picks this one.
+ * The reference has no counterpart (its launch never looks at columns,
+ * KokkosLoopMapping.cpp:861-862).  The copy holds the VALUES as they are now: build
+ * again after changing val.  Selects the COLBLOCK kernel on success; SpMV calls with
+ * this plan then ignore their crd/val arguments.  Synchronises `stream`. */
+enum lapis_hip_colblock_layout {
+  LAPIS_HIP_COLBLOCK_AUTO = 0,
+  LAPIS_HIP_COLBLOCK_WAVE = 1,
+  LAPIS_HIP_COLBLOCK_GROUP = 2
+};
 int lapis_hip_csr_plan_build_colblock(lapis_hip_csr_plan *plan, const int32_t *crd, const void *val,
-                                      int value_bytes, int slice_log2_cols, lapis_hip_stream_t stream);
+                                      int value_bytes, int layout, int slice_log2_cols,
+                                      lapis_hip_stream_t stream);
 int lapis_hip_csr_plan_destroy(lapis_hip_csr_plan *plan);
 
 /* ---- SpMV ------------------------------------------------------------------ */

@@ -200,9 +200,153 @@ __global__ __launch_bounds__(256) void colblock_low_word_kernel(long long n, con
   if (i < n) out[i] = (unsigned)keys[i];
 }
 
+
+// ---- workgroup-blocked variant -------------------------------------------------
+// One WORKGROUP per block of `rows_per_block` rows (16 per thread: 16384 rows for
+// 1024 threads), row sums in LDS shared by the whole group.  The entries of one
+// tile (row block x slice of x) are stored in COLUMN order, and the threads of the
+// group take them 64 neighbours per wavefront: with about as many entries in a tile
+// as the slice has 128-byte lines, neighbouring lanes fall into the same lines (the
+// address unit merges them into one request) and the wavefronts of the group reuse
+// each other's lines in the CU's vector cache.  Measured on a 1 MB window of
+// doubles: 430 G gathers/s in this order against 205 G/s in random order, which is
+// the request rate of L2.
+//
+// Entry word = (row within the block << slice_log2) | column within the slice;
+// tile_ptr[block * (nslices + 1) + s] is where slice s of the block starts.
+// Different wavefronts add to the same row sums with LDS atomics, so the order of
+// the additions of one row, and with it the last bits of the result, can differ
+// from run to run.
+template <typename T, int THREADS, int U, bool NT>
+__global__ __launch_bounds__(THREADS) void spmv_colgroup_kernel(int nrows, int rows_per_block, int nslices,
+                                                                int slice_log2, const int *__restrict__ tile_ptr,
+                                                                const unsigned *__restrict__ bidx,
+                                                                const T *__restrict__ bval, const T *__restrict__ x,
+                                                                T *__restrict__ y) {
+  extern __shared__ __align__(16) unsigned char colgroup_lds[];
+  T *acc = reinterpret_cast<T *>(colgroup_lds);
+  const int tid = threadIdx.x;
+  const long long row0 = (long long)blockIdx.x * rows_per_block;
+  const int rows_here = (int)std::min<long long>(rows_per_block, nrows - row0);
+  for (int i = tid; i < rows_per_block; i += THREADS) acc[i] = T(0);
+  __syncthreads();
+
+  const int *tp = tile_ptr + (long long)blockIdx.x * (nslices + 1);
+  const unsigned cmask = (1u << slice_log2) - 1u;
+  constexpr int TRIP = U * THREADS;
+  const int first = tp[0];
+  // A trip is up to TRIP consecutive entries of ONE tile, [off, min(off + TRIP, end)):
+  // the slice, and with it the base of the gathers, is uniform over the workgroup.
+  // (Trips running across tile borders, and a third trip's gathers kept in flight,
+  // both measured 10-30 % slower.)
+  int s = 0, off = first, end = tp[1];
+  while (off >= end && s + 1 < nslices) {
+    ++s;
+    end = tp[s + 1];
+  }
+  bool have = off < end;
+  unsigned ci[U];
+  T cv[U];
+  auto load_trip = [&](int o, int e, unsigned (&li)[U], T (&lv)[U]) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int p = o + u * THREADS + tid;
+      if (p < e) {
+        li[u] = ldv<NT>(bidx + p);
+        lv[u] = ldv<NT>(bval + p);
+      }
+    }
+  };
+  if (have) load_trip(off, end, ci, cv);
+  while (have) {
+    int ns = s, noff = off + TRIP, nend = end;
+    while (noff >= nend && ns + 1 < nslices) {  // tile finished: the next one starts where it ends
+      ++ns;
+      noff = nend;
+      nend = tp[ns + 1];
+    }
+    const bool more = noff < nend;
+    unsigned ni[U];
+    T nv[U];
+    if (more) load_trip(noff, nend, ni, nv);  // in flight while this trip gathers and adds
+    const T *xs = x + ((long long)s << slice_log2);
+    T pr[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (off + u * THREADS + tid < end) pr[u] = cv[u] * xs[ci[u] & cmask];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (off + u * THREADS + tid < end) lds_add(acc + (ci[u] >> slice_log2), pr[u]);
+    if (more) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        ci[u] = ni[u];
+        cv[u] = nv[u];
+      }
+    }
+    s = ns;
+    off = noff;
+    end = nend;
+    have = more;
+  }
+  __syncthreads();
+  for (int i = tid; i < rows_here; i += THREADS) y[row0 + i] = acc[i] + y[row0 + i];
+}
+
+// key = (row block << (col_bits + row_bits)) | (column << row_bits) | row in block:
+// sorted, the entries of a row block come slice by slice and by column inside a slice
+__global__ __launch_bounds__(256) void colgroup_keys_kernel(int nrows, int row_bits, int col_bits,
+                                                            const int *__restrict__ pos,
+                                                            const int *__restrict__ crd,
+                                                            unsigned long long *__restrict__ keys) {
+  const int lane = threadIdx.x & 63;
+  const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= nrows) return;
+  const unsigned long long rb = (unsigned long long)(row >> row_bits);
+  const unsigned long long rl = (unsigned long long)(row & ((1LL << row_bits) - 1));
+  const int s = pos[row], e = pos[row + 1];
+  for (int j = s + lane; j < e; j += 64) {
+    const unsigned long long c = (unsigned long long)(unsigned)crd[j];
+    keys[j] = (rb << (col_bits + row_bits)) | (c << row_bits) | rl;
+  }
+}
+
+__global__ __launch_bounds__(256) void colgroup_entry_kernel(long long n, int row_bits, int slice_log2,
+                                                             const unsigned long long *__restrict__ keys,
+                                                             unsigned *__restrict__ out) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const unsigned long long k = keys[i];
+  const unsigned rl = (unsigned)(k & ((1ull << row_bits) - 1ull));
+  const unsigned cs = (unsigned)((k >> row_bits) & ((1ull << slice_log2) - 1ull));
+  out[i] = (rl << slice_log2) | cs;
+}
+
+// tile_ptr[b * (nslices + 1) + s] = first sorted entry whose key is >= (block b, slice s)
+__global__ __launch_bounds__(256) void colgroup_tile_ptr_kernel(long long nnz, int nblocks, int nslices, int row_bits,
+                                                                int col_bits, int slice_log2,
+                                                                const unsigned long long *__restrict__ keys,
+                                                                int *__restrict__ tile_ptr) {
+  const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (t >= (long long)nblocks * (nslices + 1)) return;
+  const unsigned long long b = (unsigned long long)(t / (nslices + 1));
+  const int s = (int)(t % (nslices + 1));
+  const unsigned long long target =
+      s == nslices ? ((b + 1) << (col_bits + row_bits))
+                   : ((b << (col_bits + row_bits)) | (((unsigned long long)s << slice_log2) << row_bits));
+  long long lo = 0, hi = nnz;
+  while (lo < hi) {
+    const long long mid = (lo + hi) >> 1;
+    if (keys[mid] < target) lo = mid + 1; else hi = mid;
+  }
+  tile_ptr[t] = (int)lo;
+}
+
 void free_colblock(lapis_hip_csr_plan *p) {
   if (p->colblock_idx) (void)hipFree(p->colblock_idx);
   if (p->colblock_val) (void)hipFree(p->colblock_val);
+  if (p->colblock_tile_ptr) (void)hipFree(p->colblock_tile_ptr);
+  p->colblock_tile_ptr = nullptr;
   p->colblock_idx = nullptr;
   p->colblock_val = nullptr;
   p->colblock_built = false;
@@ -237,8 +381,53 @@ int launch_colblock_rb(const lapis_hip_csr_plan *p, const int *pos, const T *x, 
   }
 }
 
+template <typename T, int THREADS, int U, bool NT>
+int launch_colgroup_cfg(const lapis_hip_csr_plan *p, const T *x, T *y, hipStream_t st) {
+  auto kernel = spmv_colgroup_kernel<T, THREADS, U, NT>;
+  const size_t lds_bytes = sizeof(T) * (size_t)p->colblock_rows;
+  static bool attribute_set = false;  // one per instantiation; more than 64 KB of dynamic LDS has to be asked for
+  if (!attribute_set) {
+    LAPIS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    attribute_set = true;
+  }
+  const dim3 grid((unsigned)p->colblock_nblocks), block(THREADS);
+  hipEvent_t e0, e1;
+  if (timing_next_events(&e0, &e1))
+    hipExtLaunchKernelGGL(kernel, grid, block, lds_bytes, st, e0, e1, 0, (int)p->stats.nrows, p->colblock_rows,
+                          p->colblock_nslices, p->colblock_slice_log2, (const int *)p->colblock_tile_ptr,
+                          (const unsigned *)p->colblock_idx, (const T *)p->colblock_val, x, y);
+  else
+    hipLaunchKernelGGL(kernel, grid, block, lds_bytes, st, (int)p->stats.nrows, p->colblock_rows,
+                       p->colblock_nslices, p->colblock_slice_log2, (const int *)p->colblock_tile_ptr,
+                       (const unsigned *)p->colblock_idx, (const T *)p->colblock_val, x, y);
+  LAPIS_LAUNCH_CHECK();
+  return LAPIS_HIP_OK;
+}
+
+template <typename T, int THREADS>
+int launch_colgroup_threads(const lapis_hip_csr_plan *p, const T *x, T *y, hipStream_t st) {
+  const bool nt = p->nontemporal;
+  if (p->colblock_epl == 4)
+    return nt ? launch_colgroup_cfg<T, THREADS, 4, true>(p, x, y, st) : launch_colgroup_cfg<T, THREADS, 4, false>(p, x, y, st);
+  return nt ? launch_colgroup_cfg<T, THREADS, 8, true>(p, x, y, st) : launch_colgroup_cfg<T, THREADS, 8, false>(p, x, y, st);
+}
+
+template <typename T>
+int launch_colgroup(const lapis_hip_csr_plan *p, const T *x, T *y, hipStream_t st) {
+  switch (p->colblock_rows) {
+    case 16384: return launch_colgroup_threads<T, 1024>(p, x, y, st);
+    case 8192: return launch_colgroup_threads<T, 512>(p, x, y, st);
+    case 4096: return launch_colgroup_threads<T, 256>(p, x, y, st);
+    default:
+      return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT, "colblock: no workgroup kernel for %d rows per block",
+                       p->colblock_rows);
+  }
+}
+
 template <typename T>
 int launch_colblock(const lapis_hip_csr_plan *p, const int *pos, const T *x, T *y, hipStream_t st) {
+  if (p->colblock_group) return launch_colgroup<T>(p, x, y, st);
   if (p->colblock_rows == 512)
     return p->colblock_pad ? launch_colblock_rb<T, 512, 8>(p, pos, x, y, st)
                            : launch_colblock_rb<T, 512, 4>(p, pos, x, y, st);
@@ -294,7 +483,7 @@ int calibrate_pace(lapis_hip_csr_plan *p, hipStream_t st) {
     return best;
   };
   const double free_ms = time_ms(0);
-  const double entries_per_wave = (double)p->stats.nnz / (double)ceil_div(nrows, p->colblock_rows);
+  const double entries_per_wave = (double)p->stats.nnz / (double)ceil_div(nrows, p->colblock_rows);  // per row block
   unsigned best_pace = 0;
   int best_pct = 0;
   double best_ms = free_ms * 0.98;
@@ -325,10 +514,104 @@ int calibrate_pace(lapis_hip_csr_plan *p, hipStream_t st) {
   return done(LAPIS_HIP_OK);
 }
 
+
+// Builds the workgroup-blocked layout (see spmv_colgroup_kernel).
+template <typename T>
+int build_group(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int slice_log2, hipStream_t st) {
+  const int64_t nnz = p->stats.nnz, nrows = p->stats.nrows;
+  const int col_bits = std::max(1, bits_for(p->stats.ncols));
+  // 16 rows per thread; the largest block that still gives every CU one
+  int rows = 16384;
+  {
+    const char *env = getenv("LAPIS_HIP_COLBLOCK_ROWS");
+    const int want = env ? atoi(env) : 0;
+    if (want == 4096 || want == 8192 || want == 16384)
+      rows = want;
+    else
+      while (rows > 4096 && ceil_div(nrows, rows) < device_cu_count()) rows >>= 1;
+  }
+  const int row_bits = bits_for(rows);
+  slice_log2 = std::min(slice_log2, 32 - row_bits);  // an entry word holds row in block | column in slice
+  const int nblocks = (int)ceil_div(nrows, rows);
+  const int64_t nslices64 = ceil_div(p->stats.ncols, 1LL << slice_log2);
+  const int end_bit = bits_for(nblocks) + col_bits + row_bits;
+  if (end_bit > 64 || slice_log2 < 1 || nslices64 * nblocks > (1LL << 26))
+    return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT,
+                     "csr_plan_build_colblock: %d row blocks x %lld slices of 2^%d columns is not a usable tiling",
+                     nblocks, (long long)nslices64, slice_log2);
+  const int nslices = (int)nslices64;
+
+  unsigned long long *keys_in = nullptr, *keys_out = nullptr;
+  T *val_out = nullptr;
+  unsigned *idx = nullptr;
+  int *tile_ptr = nullptr;
+  void *temp = nullptr;
+  size_t temp_bytes = 0;
+  auto fail = [&](hipError_t e, const char *what) {
+    if (keys_in) (void)hipFree(keys_in);
+    if (keys_out) (void)hipFree(keys_out);
+    if (val_out) (void)hipFree(val_out);
+    if (idx) (void)hipFree(idx);
+    if (tile_ptr) (void)hipFree(tile_ptr);
+    if (temp) (void)hipFree(temp);
+    return set_error(LAPIS_HIP_ERR_RUNTIME, "csr_plan_build_colblock: %s failed: %s", what, hipGetErrorString(e));
+  };
+  hipError_t e;
+  const size_t ntiles = (size_t)nblocks * ((size_t)nslices + 1);
+  if ((e = hipMalloc(&keys_in, sizeof(unsigned long long) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
+  if ((e = hipMalloc(&keys_out, sizeof(unsigned long long) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
+  if ((e = hipMalloc(&val_out, sizeof(T) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
+  if ((e = hipMalloc(&idx, sizeof(unsigned) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
+  if ((e = hipMalloc(&tile_ptr, sizeof(int) * ntiles)) != hipSuccess) return fail(e, "hipMalloc");
+  hipLaunchKernelGGL(colgroup_keys_kernel, dim3((unsigned)ceil_div(nrows, 4)), dim3(256), 0, st, (int)nrows, row_bits,
+                     col_bits, p->pos, crd, keys_in);
+  if ((e = hipGetLastError()) != hipSuccess) return fail(e, "key kernel");
+  if ((e = hipcub::DeviceRadixSort::SortPairs(nullptr, temp_bytes, keys_in, keys_out, val, val_out, (int)nnz, 0,
+                                              end_bit, st)) != hipSuccess)
+    return fail(e, "radix sort sizing");
+  if ((e = hipMalloc(&temp, temp_bytes ? temp_bytes : 1)) != hipSuccess) return fail(e, "hipMalloc");
+  if ((e = hipcub::DeviceRadixSort::SortPairs(temp, temp_bytes, keys_in, keys_out, val, val_out, (int)nnz, 0, end_bit,
+                                              st)) != hipSuccess)
+    return fail(e, "radix sort");
+  hipLaunchKernelGGL(colgroup_entry_kernel, dim3((unsigned)ceil_div(nnz, 256)), dim3(256), 0, st, (long long)nnz,
+                     row_bits, slice_log2, keys_out, idx);
+  if ((e = hipGetLastError()) != hipSuccess) return fail(e, "entry kernel");
+  hipLaunchKernelGGL(colgroup_tile_ptr_kernel, dim3((unsigned)ceil_div((int64_t)ntiles, 256)), dim3(256), 0, st,
+                     (long long)nnz, nblocks, nslices, row_bits, col_bits, slice_log2, keys_out, tile_ptr);
+  if ((e = hipGetLastError()) != hipSuccess) return fail(e, "tile pointer kernel");
+  if ((e = hipStreamSynchronize(st)) != hipSuccess) return fail(e, "synchronize");
+  (void)hipFree(keys_in);
+  (void)hipFree(keys_out);
+  (void)hipFree(temp);
+  free_colblock(p);
+  p->colblock_group = 1;
+  {
+    const char *epl = getenv("LAPIS_HIP_COLBLOCK_EPL");
+    p->colblock_epl = epl ? atoi(epl) : 8;  // entries per thread and trip
+  }
+  p->colblock_rows = rows;
+  p->colblock_nblocks = nblocks;
+  p->colblock_nslices = nslices;
+  p->colblock_tile_ptr = tile_ptr;
+  p->colblock_idx = idx;
+  p->colblock_val = val_out;
+  p->colblock_value_bytes = (int)sizeof(T);
+  p->colblock_col_bits = col_bits;
+  p->colblock_slice_log2 = slice_log2;
+  p->colblock_built = true;
+  p->colblock_pace_fp = 0;  // the workgroups keep pace by themselves: pacing measured no gain here
+  p->colblock_free_ms = p->colblock_paced_ms = 0.0;
+  return LAPIS_HIP_OK;
+}
+
 template <typename T>
 int build(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int slice_log2, hipStream_t st) {
   const int64_t nnz = p->stats.nnz, nrows = p->stats.nrows;
   const int col_bits = std::max(1, bits_for(p->stats.ncols));
+  if (col_bits + kColblockRowBits > 32)
+    return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT,
+                     "csr_plan_build_colblock: %lld columns need %d bits, more than the %d an entry has room for",
+                     (long long)p->stats.ncols, col_bits, 32 - kColblockRowBits);
   {
     const char *rows = getenv("LAPIS_HIP_COLBLOCK_ROWS");
     p->colblock_rows = (rows && atoi(rows) == 512) ? 512 : 1024;
@@ -379,6 +662,7 @@ int build(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int slice_log
   (void)hipFree(keys_out);
   (void)hipFree(temp);
   free_colblock(p);
+  p->colblock_group = 0;
   {
     const char *stp = getenv("LAPIS_HIP_COLBLOCK_STEPS"), *epl = getenv("LAPIS_HIP_COLBLOCK_EPL"),
                *pad = getenv("LAPIS_HIP_COLBLOCK_PAD");
@@ -404,26 +688,36 @@ int build(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int slice_log
 using namespace lapis;
 
 extern "C" int lapis_hip_csr_plan_build_colblock(lapis_hip_csr_plan *plan, const int32_t *crd, const void *val,
-                                                 int value_bytes, int slice_log2_cols, lapis_hip_stream_t stream) {
+                                                 int value_bytes, int layout, int slice_log2_cols,
+                                                 lapis_hip_stream_t stream) {
   LAPIS_CHECK_INIT();
   LAPIS_REQUIRE(plan, "csr_plan_build_colblock: null plan");
   LAPIS_REQUIRE(value_bytes == 4 || value_bytes == 8, "csr_plan_build_colblock: value_bytes must be 4 or 8");
+  LAPIS_REQUIRE(layout == LAPIS_HIP_COLBLOCK_AUTO || layout == LAPIS_HIP_COLBLOCK_WAVE ||
+                    layout == LAPIS_HIP_COLBLOCK_GROUP,
+                "csr_plan_build_colblock: unknown layout %d", layout);
   const lapis_hip_csr_stats &s = plan->stats;
   LAPIS_REQUIRE(s.nnz > 0, "csr_plan_build_colblock: the matrix has no non-zeros");
   LAPIS_REQUIRE(crd && val, "csr_plan_build_colblock: null coordinates or values");
+  if (layout == LAPIS_HIP_COLBLOCK_AUTO) layout = LAPIS_HIP_COLBLOCK_GROUP;
   int col_bits = 1;
   while ((1LL << col_bits) < s.ncols) ++col_bits;
-  if (col_bits + kColblockRowBits > 32)
-    return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT,
-                     "csr_plan_build_colblock: %lld columns need %d bits, more than the %d an entry has room for",
-                     (long long)s.ncols, col_bits, 32 - kColblockRowBits);
-  if (slice_log2_cols <= 0) slice_log2_cols = value_bytes == 8 ? 17 : 18;  // 1 MB of x per slice
+  const bool group = layout == LAPIS_HIP_COLBLOCK_GROUP;
+  // default slice: 1 MB of x for the per-wavefront layout; 2 MB of fp64 / 1 MB of fp32
+  // (what an entry word has room for) for the workgroup layout
+  if (slice_log2_cols <= 0) slice_log2_cols = group ? 18 : (value_bytes == 8 ? 17 : 18);
   slice_log2_cols = std::min(slice_log2_cols, col_bits);
   hipStream_t st = as_stream(stream);
-  const int rc = value_bytes == 8 ? build<double>(plan, crd, static_cast<const double *>(val), slice_log2_cols, st)
-                                  : build<float>(plan, crd, static_cast<const float *>(val), slice_log2_cols, st);
+  int rc;
+  if (group)
+    rc = value_bytes == 8 ? build_group<double>(plan, crd, static_cast<const double *>(val), slice_log2_cols, st)
+                          : build_group<float>(plan, crd, static_cast<const float *>(val), slice_log2_cols, st);
+  else
+    rc = value_bytes == 8 ? build<double>(plan, crd, static_cast<const double *>(val), slice_log2_cols, st)
+                          : build<float>(plan, crd, static_cast<const float *>(val), slice_log2_cols, st);
   if (rc == LAPIS_HIP_OK) {
     plan->stats.kernel = LAPIS_HIP_SPMV_COLBLOCK;
+    plan->stats.colblock_layout = layout;
     plan->stats.width = 0;
     plan->stats.chunk = 0;
   }

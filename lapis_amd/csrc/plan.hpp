@@ -28,7 +28,11 @@ struct lapis_hip_csr_plan {
   int colblock_steps;        // steps per wavefront trip
   int colblock_epl;          // entries per lane per step (1, 2 or 4)
   int colblock_pad;          // 1: workgroups of 8 wavefronts instead of 4
-  int colblock_rows;         // rows per wavefront (512 or 1024)
+  int colblock_rows;         // rows per wavefront (512 or 1024), or per workgroup in the workgroup-blocked layout
+  int colblock_group;        // 1: workgroup-blocked layout (tiles in column order, row sums shared by a workgroup)
+  int colblock_nblocks;      // row blocks of the workgroup-blocked layout
+  int colblock_nslices;      // slices of x
+  int *colblock_tile_ptr;    // device, int[nblocks * (nslices + 1)]
   unsigned colblock_pace_fp; // clock ticks per entry (16.16 fixed point) of the time-triggered pacing, 0 = off
   double colblock_free_ms;   // calibration: kernel time without pacing
   double colblock_paced_ms;  // calibration: kernel time at the chosen pace

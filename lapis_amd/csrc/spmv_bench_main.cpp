@@ -209,7 +209,7 @@ int main(int argc, const char **argv) {
     CHECK_LAPIS(lapis_hip_csr_plan_create(&plan, A.nrows, A.ncols, nnz, pos, crd, 8, nullptr));
     if (kernel == "rowblock") CHECK_LAPIS(lapis_hip_csr_plan_set_kernel(plan, LAPIS_HIP_SPMV_ROWBLOCK, 0));
     else if (kernel == "nnzsplit") CHECK_LAPIS(lapis_hip_csr_plan_set_kernel(plan, LAPIS_HIP_SPMV_NNZSPLIT, 0));
-    else if (kernel == "colblock") CHECK_LAPIS(lapis_hip_csr_plan_build_colblock(plan, crd, val, 8, 0, nullptr));
+    else if (kernel == "colblock") CHECK_LAPIS(lapis_hip_csr_plan_build_colblock(plan, crd, val, 8, LAPIS_HIP_COLBLOCK_AUTO, 0, nullptr));
     else if (kernel.rfind("subwarp", 0) == 0)
       CHECK_LAPIS(lapis_hip_csr_plan_set_kernel(plan, LAPIS_HIP_SPMV_SUBWARP, atoi(kernel.c_str() + 7)));
     else if (kernel != "auto") {

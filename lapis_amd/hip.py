@@ -32,11 +32,12 @@ class CsrStats(ctypes.Structure):
                 ("mean_row_len", _dbl), ("var_row_len", _dbl), ("mean_chunk_col_span", _dbl),
                 ("reference_hint", _i64), ("reference_vector_length", ctypes.c_int32),
                 ("kernel", ctypes.c_int32), ("width", ctypes.c_int32), ("chunk", ctypes.c_int32),
-                ("colblock_recommended", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+                ("colblock_recommended", ctypes.c_int32), ("colblock_layout", ctypes.c_int32)]
 
     def as_dict(self):
         d = {k: getattr(self, k) for k, _ in self._fields_}
         d["kernel_name"] = KERNEL_NAMES.get(self.kernel, "?")
+        d["colblock_layout_name"] = {0: None, 1: "wave", 2: "group"}.get(self.colblock_layout)
         return d
 
 
@@ -51,7 +52,7 @@ _SIGNATURES = {
     "lapis_hip_csr_plan_set_kernel": [_vp, _int, _int],
     "lapis_hip_csr_plan_get_stats": [_vp, ctypes.POINTER(CsrStats)],
     "lapis_hip_csr_plan_destroy": [_vp],
-    "lapis_hip_csr_plan_build_colblock": [_vp, _vp, _vp, _int, _int, _vp],
+    "lapis_hip_csr_plan_build_colblock": [_vp, _vp, _vp, _int, _int, _int, _vp],
     "lapis_hip_spmv_csr_f64_i32": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp],
     "lapis_hip_spmv_csr_f32_i32": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp],
     "lapis_hip_spmm_csr_f32_i32": [_i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp],
@@ -150,6 +151,9 @@ def kernel_timing_stop():
     return {"count": n.value, "mean_ms": mean.value, "min_ms": mn.value, "max_ms": mx.value}
 
 
+COLBLOCK_LAYOUTS = {"auto": 0, "wave": 1, "group": 2}
+
+
 class CsrPlan:
     """Row-length statistics of one CSR matrix and the SpMV kernel chosen from them."""
 
@@ -176,10 +180,11 @@ class CsrPlan:
         check(self._lib.lapis_hip_csr_plan_set_kernel(self._handle, kernel, width))
         return self
 
-    def build_colblock(self, crd, val, slice_log2_cols=0, stream=None):
-        """Copy the matrix into the column-blocked layout and select that kernel."""
+    def build_colblock(self, crd, val, slice_log2_cols=0, layout="auto", stream=None):
+        """Copy the matrix into a column-blocked layout ("wave", "group" or "auto") and select that kernel."""
         check(self._lib.lapis_hip_csr_plan_build_colblock(self._handle, _ptr(crd), _ptr(val), val.element_size(),
-                                                          slice_log2_cols, _stream(stream)))
+                                                          COLBLOCK_LAYOUTS[layout], slice_log2_cols,
+                                                          _stream(stream)))
         return self.set_kernel(SPMV_COLBLOCK)
 
     def destroy(self):
