@@ -33,6 +33,10 @@ struct lapis_hip_csr_plan {
   int colblock_nblocks;      // row blocks of the workgroup-blocked layout
   int colblock_nslices;      // slices of x
   int *colblock_tile_ptr;    // device, int[nblocks * (nslices + 1)]
+  int colblock_nsplit;       // workgroups sharing one row block (each takes a share of the slices)
+  int colblock_long_threshold; // rows of this many entries or more are taken from the CSR arrays instead
+  int colblock_npieces;      // pieces of long rows
+  int *colblock_pieces;      // device, int[3 * npieces]: row, first entry, one past the last
   unsigned colblock_pace_fp; // clock ticks per entry (16.16 fixed point) of the time-triggered pacing, 0 = off
   double colblock_free_ms;   // calibration: kernel time without pacing
   double colblock_paced_ms;  // calibration: kernel time at the chosen pace
@@ -44,7 +48,8 @@ constexpr int kColblockRowBits = 10;
 
 // Launches the column-blocked kernel; defined in colblock.hip.
 template <typename T>
-int launch_colblock(const lapis_hip_csr_plan *plan, const int *pos, const T *x, T *y, hipStream_t st);
+int launch_colblock(const lapis_hip_csr_plan *plan, const int *pos, const int *crd, const T *val, const T *x, T *y,
+                    hipStream_t st);
 void free_colblock(lapis_hip_csr_plan *plan);
 
 // y = A x without reading y; defined in spmv.hip.

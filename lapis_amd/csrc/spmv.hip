@@ -551,7 +551,8 @@ int spmv_impl(lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, const int3
                      (long long)s.nrows, (long long)s.ncols, (const void *)plan->pos, (long long)nrows,
                      (long long)ncols, (const void *)pos);
   if (s.nnz == 0) return LAPIS_HIP_OK;
-  LAPIS_REQUIRE(crd && val && x, "spmv: null coordinates, values or x with %lld non-zeros", (long long)s.nnz);
+  LAPIS_REQUIRE(x && (s.kernel == LAPIS_HIP_SPMV_COLBLOCK || (crd && val)),
+                "spmv: null coordinates, values or x with %lld non-zeros", (long long)s.nnz);
   const bool vec = aligned16(crd) && aligned16(val);
   const bool nt = plan->nontemporal;
   switch (s.kernel) {
@@ -572,7 +573,7 @@ int spmv_impl(lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, const int3
       if (!plan->colblock_built || plan->colblock_value_bytes != (int)sizeof(T))
         return set_error(LAPIS_HIP_ERR_PLAN_MISMATCH, "spmv: the plan holds no column-blocked copy for %d-byte values",
                          (int)sizeof(T));
-      return launch_colblock<T>(plan, pos, x, y, st);
+      return launch_colblock<T>(plan, pos, crd, val, x, y, st);
     default:
       return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT, "spmv: plan holds unknown kernel %d", s.kernel);
   }
@@ -675,16 +676,9 @@ extern "C" int lapis_hip_csr_plan_create(lapis_hip_csr_plan **out, int64_t nrows
   s.var_row_len = nrows ? std::max(0.0, host.sum_sq / (double)nrows - s.mean_row_len * s.mean_row_len) : 0.0;
   s.mean_chunk_col_span = (crd && nnz > 0) ? (double)host.span_sum / (double)ceil_div(nnz, 1024) : -1.0;
   // The column-blocked copy pays when the gathers of a chunk wander over more of x
-  // than an XCD's L2 keeps (4 MB, shared with the streamed arrays), the rows are even
-  // enough for equal row blocks to mean equal work, and the entry encoding fits.
-  {
-    int col_bits = 1;
-    while ((1LL << col_bits) < ncols) ++col_bits;
-    s.colblock_recommended = (s.mean_chunk_col_span * value_bytes > 2.0 * 1024 * 1024 && col_bits <= 22 &&
-                              nnz >= (1 << 20) && (double)s.max_row_len <= 64.0 * std::max(1.0, s.mean_row_len))
-                                 ? 1
-                                 : 0;
-  }
+  // than an XCD's L2 keeps (4 MB, shared with the streamed arrays) and the matrix is
+  // large enough for the extra launch work not to matter.
+  s.colblock_recommended = (s.mean_chunk_col_span * value_bytes > 2.0 * 1024 * 1024 && nnz >= (1 << 20)) ? 1 : 0;
   s.reference_hint = reference_hint(nrows, ends[0], ends[1]);
   s.reference_vector_length = reference_vector_length(s.reference_hint);
   p->pos = pos;
