@@ -506,10 +506,15 @@ int launch_colgroup_cfg(const lapis_hip_csr_plan *p, const int *crd, const T *va
     attribute_set = true;
   }
   const dim3 grid((unsigned)(p->colblock_nblocks * p->colblock_nsplit)), block(THREADS);
-  hipEvent_t e0, e1;
-  if (timing_next_events(&e0, &e1))
-    hipExtLaunchKernelGGL(kernel, grid, block, lds_bytes, st, e0, e1, 0, (int)p->stats.nrows, p->colblock_rows,
-                          p->colblock_nslices, p->colblock_nsplit, p->colblock_slice_log2,
+  const bool pieces = p->colblock_npieces > 0;
+  if (pieces) LAPIS_REQUIRE(crd && val, "spmv: this plan takes its long rows from crd/val, which are null");
+  // kernel timing covers the whole product: from the start of the blocked kernel to the
+  // end of the long-row kernel when there is one
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  const bool timed = timing_next_events(&e0, &e1);
+  if (timed)
+    hipExtLaunchKernelGGL(kernel, grid, block, lds_bytes, st, e0, pieces ? nullptr : e1, 0, (int)p->stats.nrows,
+                          p->colblock_rows, p->colblock_nslices, p->colblock_nsplit, p->colblock_slice_log2,
                           (const int *)p->colblock_tile_ptr, (const unsigned *)p->colblock_idx,
                           (const T *)p->colblock_val, x, y);
   else
@@ -518,10 +523,14 @@ int launch_colgroup_cfg(const lapis_hip_csr_plan *p, const int *crd, const T *va
                        (const int *)p->colblock_tile_ptr, (const unsigned *)p->colblock_idx,
                        (const T *)p->colblock_val, x, y);
   LAPIS_LAUNCH_CHECK();
-  if (p->colblock_npieces > 0) {
-    LAPIS_REQUIRE(crd && val, "spmv: this plan takes its long rows from crd/val, which are null");
-    hipLaunchKernelGGL(spmv_long_piece_kernel<T>, dim3((unsigned)p->colblock_npieces), dim3(256), 0, st,
-                       (const int *)p->colblock_pieces, crd, val, x, y);
+  if (pieces) {
+    const dim3 pgrid((unsigned)p->colblock_npieces), pblock(256);
+    if (timed)
+      hipExtLaunchKernelGGL(spmv_long_piece_kernel<T>, pgrid, pblock, 0, st, nullptr, e1, 0,
+                            (const int *)p->colblock_pieces, crd, val, x, y);
+    else
+      hipLaunchKernelGGL(spmv_long_piece_kernel<T>, pgrid, pblock, 0, st, (const int *)p->colblock_pieces, crd, val, x,
+                         y);
     LAPIS_LAUNCH_CHECK();
   }
   return LAPIS_HIP_OK;
