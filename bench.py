@@ -140,6 +140,22 @@ def run_spmv(args, cfg):
                      "traffic": traffic_from_profiles("%s_config%d" % (family, cfg)) if cfg else None,
                      "kernel_ms_mean": kt["mean_ms"], "kernel_ms_min": kt["min_ms"], "launches_timed": kt["count"]},
     }
+    if args.host_buffers:
+        # The generated-module entry takes HOST arrays (the reference's Python path):
+        # every call uploads the matrix and vectors and copies y back.  Reported beside
+        # `value`, never as it.
+        from lapis_amd.module import LAPISModule
+        mod = LAPISModule()
+        spec = ((A.nrows, A.ncols), (A.nrows + 1, A.nnz, A.nnz))
+        yh = np.zeros(A.nrows, dtype=dtype)
+        mod.spmv(A.pos, A.crd, A.val, spec, x, yh)  # warm-up
+        reps = 3
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            mod.spmv(A.pos, A.crd, A.val, spec, x, yh)
+        hms = (time.perf_counter() - t0) / reps * 1e3
+        out["host_buffers"] = {"entry": "py_spmv via LAPISModule.spmv (host arrays, H2D + kernel + D2H per call)",
+                               "ms_per_call": hms, "GB/s": bytes_step / (hms * 1e-3) / 1e9}
     if published:
         # fenced per-call protocol of the published numbers: one call, one synchronise
         t0 = time.perf_counter()
@@ -279,6 +295,8 @@ def main():
                     help="layout of the column-blocked copy (auto = group)")
     ap.add_argument("--width", type=int, default=0, help="lanes per row with --kernel subwarp (0 = the reference's rule)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--host-buffers", action="store_true",
+                    help="also time the generated-module entry point, which takes host arrays (PCIe-inclusive)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch the library's copy kernel on 1 GiB three times, the known-size reference "
                          "that rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")

@@ -9,11 +9,15 @@
 // r.z at the top of an iteration is the rz' of the one before (same vectors), so
 // it is carried instead of recomputed; without a preconditioner z is r and rz' is rr.
 //
-// Every dot product is two launches: the vector kernel leaves one partial per block,
-// a one-block kernel behind it adds the partials in index order and updates the
-// scalars.  Kernel boundaries order the two, so no block ever needs a device-scope
-// fence (on a multi-XCD part such a fence writes back and invalidates L2, and two
-// thousand of them per kernel cost more than the vector pass itself).
+// A dot product never needs a launch of its own: the vector kernel that produces the
+// operands leaves one partial per block, and EVERY block of the next vector kernel
+// adds those partials (at most 2048 doubles, from L2) in index order before it
+// starts, so all blocks hold the same bits of alpha, beta and relres.  Kernel
+// boundaries do the ordering; no block needs a device-scope fence (on a multi-XCD
+// part such a fence writes back and invalidates L2, and two thousand of them per
+// kernel cost more than the vector pass itself).  The iteration number is a kernel
+// argument (the host knows which iteration it is queueing); scalars that one kernel
+// both reads and replaces (r.z) are kept twice, indexed by iteration parity.
 #include <algorithm>
 #include <cmath>
 
@@ -24,17 +28,15 @@
 namespace lapis {
 
 struct CgState {
-  double pAp;      // p . Ap
-  double rz;       // r . z of the current residual
-  double rz_next;  // r . z after the update
+  double pAp;      // p . Ap of the last iteration (diagnostic)
+  double rz[2];    // r . z entering iteration i is rz[i & 1]
   double rr;       // r . r after the update
   double initres;  // sqrt(r0 . r0)
   double relres;
-  unsigned long long iter;  // the reference's counter i (starts at 1)
+  unsigned long long iter;  // the reference's counter i at exit (it starts at 1)
   unsigned long long maxiter;
   double tol;
   int done;
-  int roll_pending;  // update_p has run: rz = rz_next and i = i+1 are due
 };
 
 __device__ __forceinline__ double block_sum_256d(double v, double *lds4) {
@@ -44,6 +46,18 @@ __device__ __forceinline__ double block_sum_256d(double v, double *lds4) {
   const double total = ((lds4[0] + lds4[1]) + lds4[2]) + lds4[3];
   __syncthreads();
   return total;
+}
+
+// The exit flag, read once per block: block 0 of the kernel that makes the convergence
+// test raises it while other blocks of the same kernel may still be starting, and
+// every thread of a block has to take the same way past the barriers below.
+__device__ __forceinline__ bool block_sees_done(const CgState *st) {
+  __shared__ int seen;
+  if (threadIdx.x == 0) seen = st->done;
+  __syncthreads();
+  const bool d = seen != 0;
+  __syncthreads();
+  return d;
 }
 
 // Sum of partials[0..count) in a fixed order, by one block of 256 threads.
@@ -105,15 +119,20 @@ __global__ __launch_bounds__(256) void cg_pap_kernel(long long n, const double *
   if (threadIdx.x == 0) partials[blockIdx.x] = bsum;
 }
 
-// x += alpha p ; r -= alpha Ap ; block partials of r.r
+// x += alpha p ; r -= alpha Ap ; block partials of r.r.   alpha = r.z / p.Ap with p.Ap
+// summed here from the partials the p.Ap kernel left.
 __global__ __launch_bounds__(256) void cg_update_xr_kernel(long long n, const double *__restrict__ p,
                                                            const double *__restrict__ Ap, double *__restrict__ x,
-                                                           double *__restrict__ r, const CgState *st,
-                                                           double *__restrict__ partials, int vec) {
+                                                           double *__restrict__ r, CgState *st,
+                                                           unsigned long long iter, int count,
+                                                           const double *__restrict__ pap_partials,
+                                                           double *__restrict__ rr_partials, int vec) {
   __shared__ double lds4[4];
-  if (st->done) return;
-  const double alpha = st->rz / st->pAp;
+  if (block_sees_done(st)) return;
+  const double pAp = ordered_total(pap_partials, count, lds4);
+  const double alpha = st->rz[iter & 1] / pAp;
   const double malpha = -alpha;
+  if (blockIdx.x == 0 && threadIdx.x == 0) st->pAp = pAp;
   double rr = 0.0;
   const long long nv = vec ? n / 2 : 0;
   CG_GRID_STRIDE(i, 0, nv) {
@@ -138,16 +157,35 @@ __global__ __launch_bounds__(256) void cg_update_xr_kernel(long long n, const do
     rr = rr + ri * ri;
   }
   const double bsum = block_sum_256d(rr, lds4);
-  if (threadIdx.x == 0) partials[blockIdx.x] = bsum;
+  if (threadIdx.x == 0) rr_partials[blockIdx.x] = bsum;
 }
 
-// z = r * dinv ; block partials of r.z     (preconditioned runs only)
+// The convergence test of examples/pcg_solve.py:84-90, made by every block from the
+// r.r partials: leave when !(relres > tol) or i == maxiter.  Block 0 records the exit.
+__device__ __forceinline__ bool cg_continues(CgState *st, unsigned long long iter, double rr) {
+  const double relres = sqrt(rr) / st->initres;
+  const bool go_on = (relres > st->tol) && (iter != st->maxiter);
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    st->rr = rr;
+    st->relres = relres;
+    if (!go_on) {
+      st->iter = iter;
+      st->done = 1;
+    }
+  }
+  return go_on;
+}
+
+// Convergence test, then z = r * dinv (or r / dinv) ; block partials of r.z     (preconditioned runs only)
 __global__ __launch_bounds__(256) void cg_precond_kernel(long long n, const double *__restrict__ r,
                                                          const double *__restrict__ dinv, double *__restrict__ z,
-                                                         const CgState *st, double *__restrict__ partials, int vec,
-                                                         int divide) {
+                                                         CgState *st, unsigned long long iter, int count,
+                                                         const double *__restrict__ rr_partials,
+                                                         double *__restrict__ rz_partials, int vec, int divide) {
   __shared__ double lds4[4];
-  if (st->done) return;
+  if (block_sees_done(st)) return;
+  const double rr = ordered_total(rr_partials, count, lds4);
+  if (!cg_continues(st, iter, rr)) return;
   double acc = 0.0;
   const long long nv = vec ? n / 2 : 0;
   CG_GRID_STRIDE(i, 0, nv) {
@@ -166,7 +204,7 @@ __global__ __launch_bounds__(256) void cg_precond_kernel(long long n, const doub
     acc = acc + ri * zi;
   }
   const double bsum = block_sum_256d(acc, lds4);
-  if (threadIdx.x == 0) partials[blockIdx.x] = bsum;
+  if (threadIdx.x == 0) rz_partials[blockIdx.x] = bsum;
 }
 
 // Elementwise pieces of the masked operator and of the moment right-hand sides
@@ -191,11 +229,20 @@ __global__ __launch_bounds__(256) void normalize_mom2_kernel(long long n, const 
   }
 }
 
-// p = z + beta p with beta = rz_next/rz.
+// p = z + beta p with beta = (new r.z) / (old r.z).  Unpreconditioned, z is r and the
+// new r.z is r.r: this kernel then makes the convergence test itself; preconditioned,
+// the test was made by cg_precond_kernel and `partials` holds r.z.
 __global__ __launch_bounds__(256) void cg_update_p_kernel(long long n, const double *__restrict__ z,
-                                                          double *__restrict__ p, const CgState *st, int vec) {
-  if (st->done) return;
-  const double beta = st->rz_next / st->rz;
+                                                          double *__restrict__ p, CgState *st,
+                                                          unsigned long long iter, int count,
+                                                          const double *__restrict__ partials, int preconditioned,
+                                                          int vec) {
+  __shared__ double lds4[4];
+  if (block_sees_done(st)) return;
+  const double rz_new = ordered_total(partials, count, lds4);
+  if (!preconditioned && !cg_continues(st, iter, rz_new)) return;
+  const double beta = rz_new / st->rz[iter & 1];
+  if (blockIdx.x == 0 && threadIdx.x == 0) st->rz[(iter + 1) & 1] = rz_new;
   const long long nv = vec ? n / 2 : 0;
   CG_GRID_STRIDE(i, 0, nv) {
     const v2d zv = ld2(z, i);
@@ -210,48 +257,17 @@ __global__ __launch_bounds__(256) void cg_update_p_kernel(long long n, const dou
   }
 }
 
-// The one-block kernels that turn block partials into scalars.
-enum { kStageInit = 0, kStagePap = 1, kStageResidual = 2, kStagePrecond = 3 };
-
-__global__ __launch_bounds__(256) void cg_scalar_kernel(int stage, int count, const double *__restrict__ partials,
-                                                        CgState *st, int preconditioned) {
+// One block, once per solve: the scalars of the initial residual.
+__global__ __launch_bounds__(256) void cg_init_scalar_kernel(int count, const double *__restrict__ partials,
+                                                             CgState *st) {
   __shared__ double lds4[4];
-  if (stage == kStageInit) {
-    const double trr = ordered_total(partials, count, lds4);
-    const double trz = ordered_total(partials + kDotMaxBlocks, count, lds4);
-    if (threadIdx.x == 0) {
-      st->initres = sqrt(trr);
-      st->rz = trz;
-      st->iter = 1;
-      st->done = 0;
-      st->roll_pending = 0;
-    }
-    return;
-  }
-  if (st->done) return;
-  const double total = ordered_total(partials, count, lds4);
-  if (threadIdx.x != 0) return;
-  if (stage == kStagePap) {
-    // the first scalar step of an iteration also rolls the previous one forward:
-    // update_p of that iteration has read rz and rz_next by now
-    if (st->roll_pending) {
-      st->rz = st->rz_next;
-      st->iter = st->iter + 1;
-      st->roll_pending = 0;
-    }
-    st->pAp = total;
-  } else if (stage == kStageResidual) {
-    const double relres = sqrt(total) / st->initres;
-    st->rr = total;
-    st->relres = relres;
-    if (!preconditioned) st->rz_next = total;
-    const bool go_on = (relres > st->tol) && (st->iter != st->maxiter);
-    if (go_on)
-      st->roll_pending = 1;
-    else
-      st->done = 1;
-  } else {
-    st->rz_next = total;
+  const double trr = ordered_total(partials, count, lds4);
+  const double trz = ordered_total(partials + kDotMaxBlocks, count, lds4);
+  if (threadIdx.x == 0) {
+    st->initres = sqrt(trr);
+    st->rz[1] = trz;  // the first iteration is i = 1
+    st->iter = 1;
+    st->done = 0;
   }
 }
 
@@ -329,7 +345,7 @@ int pcg_run(lapis_hip_csr_plan *plan, int64_t n, const int32_t *pos, const int32
   double *tmp = mask ? work + 4 * stride : nullptr;
   const int divide = mask ? 1 : 0;
   PCG_TRY(hipMalloc(&state, sizeof(CgState)));
-  PCG_TRY(hipMalloc(&partials, sizeof(double) * 2 * kDotMaxBlocks));
+  PCG_TRY(hipMalloc(&partials, sizeof(double) * 3 * kDotMaxBlocks));
   CgState h{};
   h.maxiter = maxiter;
   h.tol = tol;
@@ -343,8 +359,9 @@ int pcg_run(lapis_hip_csr_plan *plan, int64_t n, const int32_t *pos, const int32
                       : 0;
   hipLaunchKernelGGL(cg_init_kernel, dim3(grid), dim3(256), 0, st, (long long)n, b, dinv, x, r, z, p, partials,
                      divide);
-  hipLaunchKernelGGL(cg_scalar_kernel, dim3(1), dim3(256), 0, st, (int)kStageInit, grid, partials, state, pre);
+  hipLaunchKernelGGL(cg_init_scalar_kernel, dim3(1), dim3(256), 0, st, grid, partials, state);
   PCG_TRY(hipGetLastError());
+  double *pap_partials = partials, *rr_partials = partials + kDotMaxBlocks, *rz_partials = partials + 2 * kDotMaxBlocks;
 
   // The host looks at the device's `done` flag after each batch of iterations; a
   // batch queued past convergence costs launches only (its kernels return at once
@@ -374,19 +391,15 @@ int pcg_run(lapis_hip_csr_plan *plan, int64_t n, const int32_t *pos, const int32
         // Ap = A p: the reference zero-fills Ap and accumulates (examples/pcg_solve.py:12-19)
         PCG_RC(spmv_overwrite_f64(plan, n, n, pos, crd, val, p, Ap, stream));
       }
-      hipLaunchKernelGGL(cg_pap_kernel, dim3(grid), dim3(256), 0, st, (long long)n, p, Ap, partials, vec);
-      hipLaunchKernelGGL(cg_scalar_kernel, dim3(1), dim3(256), 0, st, (int)kStagePap, grid, partials, state, pre);
-      hipLaunchKernelGGL(cg_update_xr_kernel, dim3(grid), dim3(256), 0, st, (long long)n, p, Ap, x, r, state,
-                         partials, vec);
-      hipLaunchKernelGGL(cg_scalar_kernel, dim3(1), dim3(256), 0, st, (int)kStageResidual, grid, partials, state,
-                         pre);
-      if (pre) {
-        hipLaunchKernelGGL(cg_precond_kernel, dim3(grid), dim3(256), 0, st, (long long)n, r, dinv, z, state,
-                           partials, vec, divide);
-        hipLaunchKernelGGL(cg_scalar_kernel, dim3(1), dim3(256), 0, st, (int)kStagePrecond, grid, partials, state,
-                           pre);
-      }
-      hipLaunchKernelGGL(cg_update_p_kernel, dim3(grid), dim3(256), 0, st, (long long)n, z, p, state, vec);
+      const unsigned long long iter = launched + (uint64_t)it + 1;  // the reference's counter for this pass
+      hipLaunchKernelGGL(cg_pap_kernel, dim3(grid), dim3(256), 0, st, (long long)n, p, Ap, pap_partials, vec);
+      hipLaunchKernelGGL(cg_update_xr_kernel, dim3(grid), dim3(256), 0, st, (long long)n, p, Ap, x, r, state, iter,
+                         grid, pap_partials, rr_partials, vec);
+      if (pre)
+        hipLaunchKernelGGL(cg_precond_kernel, dim3(grid), dim3(256), 0, st, (long long)n, r, dinv, z, state, iter,
+                           grid, rr_partials, rz_partials, vec, divide);
+      hipLaunchKernelGGL(cg_update_p_kernel, dim3(grid), dim3(256), 0, st, (long long)n, z, p, state, iter, grid,
+                         pre ? rz_partials : rr_partials, pre, vec);
       PCG_TRY(hipGetLastError());
     }
     launched += (uint64_t)todo;
