@@ -53,6 +53,22 @@ LAPIS_DECLARE_MEMREF_1D(lapis_memref_1d_f32, float);
 LAPIS_DECLARE_MEMREF_2D(lapis_memref_2d_f32, float);
 LAPIS_DECLARE_MEMREF_2D(lapis_memref_2d_f64, double);
 
+/* StridedMemRefType<T,3> */
+typedef struct lapis_memref_3d_f32 {
+  float *basePtr;
+  float *data;
+  int64_t offset;
+  int64_t sizes[3];
+  int64_t strides[3];
+} lapis_memref_3d_f32;
+
+/* storage specifier of a decomposed 3-D CSRV tensor (dense, compressed, dense):
+ * ((n1, n2, nh), (n1+1, nnz, nnz*nh)) as examples/bspmm.py:103 passes it */
+typedef struct lapis_csrv_specifier {
+  int64_t dimSizes[3];
+  int64_t memSizes[3];
+} lapis_csrv_specifier;
+
 /* storage specifier of a decomposed 2-D CSR tensor (benchmarks/spmv/main.cpp:48-51) */
 typedef struct lapis_csr_specifier {
   int64_t dimSizes[2];
@@ -91,6 +107,11 @@ void py_spmm(lapis_memref_2d_f32 **ret0, lapis_memref_1d_i32 *pos, lapis_memref_
 void py_spmm_f64(lapis_memref_2d_f64 **ret0, lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd,
                  lapis_memref_1d_f64 *val, const lapis_csr_specifier *spec, lapis_memref_2d_f64 *B,
                  lapis_memref_2d_f64 *C);
+
+/* func @pte_local_bspmm(A: ?x?x?xf32 #csrv, B: ?x?x?xf32) -> ?x?x?xf32 of examples/bspmm.py:26-52:
+ * out(i, d, h) = sum_c A(i, c, h) * B(c, d, h); the result is allocated and zero-filled inside. */
+void py_pte_local_bspmm(lapis_memref_3d_f32 **ret0, lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd,
+                        lapis_memref_1d_f32 *val, const lapis_csrv_specifier *spec, lapis_memref_3d_f32 *B);
 
 /* func @plus_norm(x, y) -> (x+y, ||x+y||) of examples/multiple_results.py:8-19. */
 void py_plus_norm(lapis_memref_1d_f64 **ret0, double *ret1, lapis_memref_1d_f64 *x, lapis_memref_1d_f64 *y);

@@ -280,6 +280,46 @@ extern "C" void py_spmm_f64(lapis_memref_2d_f64 **ret0, lapis_memref_1d_i32 *pos
   spmm_entry<double>(ret0, pos, crd, val, spec, B, C);
 }
 
+extern "C" void py_pte_local_bspmm(lapis_memref_3d_f32 **ret0, lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd,
+                                   lapis_memref_1d_f32 *val, const lapis_csrv_specifier *spec,
+                                   lapis_memref_3d_f32 *B) {
+  int32_t *hpos = host_data(pos, 1, "positions");
+  int32_t *hcrd = host_data(crd, 1, "coordinates");
+  float *hval = host_data(val, 1, "values");
+  float *hB = host_data(B, 3, "B");
+  const int64_t n1 = spec->dimSizes[0], n2 = spec->dimSizes[1], nh = spec->dimSizes[2];
+  const int64_t nnz = spec->memSizes[1];
+  const int64_t dh = B->sizes[1];
+  if (n1 < 0 || n2 < 0 || nh < 0 || nnz < 0 || spec->memSizes[0] != n1 + 1 || spec->memSizes[2] != nnz * nh ||
+      pos->sizes[0] < n1 + 1 || crd->sizes[0] < nnz || val->sizes[0] < nnz * nh)
+    module_abort("bspmm: storage specifier and buffers do not agree");
+  if (B->sizes[0] < n2 || B->sizes[2] != nh) module_abort("bspmm: operand shapes do not agree");
+  const size_t out_count = (size_t)(n1 * dh * nh);
+  float *hout = static_cast<float *>(keep_alive_alloc(sizeof(float) * out_count));
+  memset(hout, 0, sizeof(float) * out_count);  // linalg.fill of the result (examples/bspmm.py:40-42)
+  if (out_count > 0) {
+    DeviceMirror<int32_t> dpos(hpos, (size_t)n1 + 1), dcrd(hcrd, (size_t)nnz);
+    DeviceMirror<float> dval(hval, (size_t)(nnz * nh)), dB(hB, (size_t)(n2 * dh * nh)), dout(hout, out_count);
+    // the plan is built only for its structure check: a bad coordinate must not reach the kernel
+    lapis_hip_csr_plan *plan = nullptr;
+    check(lapis_hip_csr_plan_create(&plan, n1, n2, nnz, dpos.dev, dcrd.dev, 4, nullptr), "lapis_hip_csr_plan_create");
+    lapis_hip_csr_plan_destroy(plan);
+    check(lapis_hip_bspmm_csrv_f32_i32(n1, n2, dh, nh, dpos.dev, dcrd.dev, dval.dev, dB.dev, dout.dev, nullptr),
+          "lapis_hip_bspmm_csrv_f32_i32");
+    check(lapis_hip_stream_synchronize(nullptr), "stream synchronize");
+    dout.sync_host();
+  }
+  (*ret0)->basePtr = hout;
+  (*ret0)->data = hout;
+  (*ret0)->offset = 0;
+  (*ret0)->sizes[0] = n1;
+  (*ret0)->sizes[1] = dh;
+  (*ret0)->sizes[2] = nh;
+  (*ret0)->strides[0] = dh * nh;
+  (*ret0)->strides[1] = nh;
+  (*ret0)->strides[2] = 1;
+}
+
 extern "C" void py_plus_norm(lapis_memref_1d_f64 **ret0, double *ret1, lapis_memref_1d_f64 *x,
                              lapis_memref_1d_f64 *y) {
   double *hx = host_data(x, 1, "x");

@@ -128,6 +128,24 @@ class LAPISModule:
               ctypes.pointer(rt.get_ranked_memref_descriptor(param5)))
         return (rt.ranked_memref_to_numpy(ret0[0]))
 
+    # func @pte_local_bspmm(A: CSRV, B) -> out      (examples/bspmm.py:26-52, called at :103)
+    def pte_local_bspmm(self, param0, param1, param2, param3, param4):
+        param0 = numpy.require(param0, dtype=numpy.int32, requirements=['C'])
+        param1 = numpy.require(param1, dtype=numpy.int32, requirements=['C'])
+        param2 = numpy.require(param2, dtype=numpy.float32, requirements=['C'])
+        spec = numpy.zeros(6, dtype=numpy.int64)  # ((n1, n2, nh), (n1+1, nnz, nnz*nh)) flattened
+        spec[0:3] = param3[0]
+        spec[3:6] = param3[1]
+        param4 = numpy.require(param4, dtype=numpy.float32, requirements=['C'])
+        ret0 = ctypes.pointer(ctypes.pointer(rt.make_nd_memref_descriptor(3, ctypes.c_float)()))
+        self.libHandle.py_pte_local_bspmm(ret0,
+                                          ctypes.pointer(rt.get_ranked_memref_descriptor(param0)),
+                                          ctypes.pointer(rt.get_ranked_memref_descriptor(param1)),
+                                          ctypes.pointer(rt.get_ranked_memref_descriptor(param2)),
+                                          spec.ctypes.data_as(ctypes.c_void_p),
+                                          ctypes.pointer(rt.get_ranked_memref_descriptor(param4)))
+        return (rt.ranked_memref_to_numpy(ret0[0]))
+
     # func @plus_norm(x, y) -> (x+y, norm)      (examples/multiple_results.py:8,34)
     def plus_norm(self, param0, param1):
         param0 = numpy.require(param0, dtype=numpy.float64, requirements=['C'])

@@ -21,8 +21,8 @@ module {
 
 
 def test_public_functions_skip_private_helpers():
-    assert [n for n, _ in _public_functions(PCG)] == ["pcg"]
-    assert [n for n, _ in _public_functions(SPMV_NOALLOC)] == ["spmv"]
+    assert [f[0] for f in _public_functions(PCG)] == ["pcg"]
+    assert [f[0] for f in _public_functions(SPMV_NOALLOC)] == ["spmv"]
 
 
 def test_bind_accepts_the_path_and_renames_main():
@@ -31,6 +31,24 @@ def test_bind_accepts_the_path_and_renames_main():
     assert b.bind(PCG) == ["pcg"]
     torch_mv = "func.func @main(%arg0: tensor<5x5xf64, #sparse>, %arg1: tensor<5xf64>) -> tensor<5xf64> { }"
     assert b.bind(torch_mv) == ["lapis_main"]
+
+
+BSPMM = """
+#csrv = #sparse_tensor.encoding<{ map = (d0, d1, d2) -> (d0 : dense, d1 : compressed, d2 : dense), posWidth = 32, crdWidth = 32}>
+module {
+  func.func @pte_local_bspmm(%A: tensor<?x?x?xf32, #csrv>,
+    %B: tensor<?x?x?xf32>) ->  tensor<?x?x?xf32>
+  { }
+  func.func @print_csrv(%A: tensor<?x?x?xf32, #csrv>)
+  { }
+}"""
+
+
+def test_bind_takes_the_batched_csrv_product_and_sets_its_print_helper_aside():
+    # shape of the module in examples/bspmm.py:10-60
+    b = KokkosBackend(decompose_tensors=True)
+    assert b.bind(BSPMM) == ["pte_local_bspmm"]
+    assert b.unbound == ["print_csrv"]
 
 
 def test_bind_rejects_what_the_module_does_not_implement():
