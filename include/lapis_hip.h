@@ -96,9 +96,10 @@ typedef struct lapis_hip_csr_stats {
   int32_t kernel;      /* enum lapis_hip_spmv_kernel, never AUTO */
   int32_t width;       /* lanes per row for SUBWARP, else 0 */
   int32_t chunk;       /* non-zeros per wavefront for NNZSPLIT (512, 1024 or 2048), else 0 */
-  /* 1 if lapis_hip_csr_plan_build_colblock is expected to pay for this matrix (x far
-   * larger than an XCD's L2, gathers spread all over it, even rows); plan creation
-   * cannot build it itself because it is not given the values */
+  /* 1 if lapis_hip_csr_plan_build_colblock is expected to pay for this matrix (the
+   * gathers of a 1024-non-zero chunk range over more of x than an XCD's L2 keeps, and
+   * the matrix has at least 2^20 non-zeros); plan creation cannot build the copy
+   * itself because it is not given the values */
   int32_t colblock_recommended;
   /* enum lapis_hip_colblock_layout of the copy this plan holds, 0 if none */
   int32_t colblock_layout;
@@ -136,11 +137,16 @@ int lapis_hip_csr_plan_get_stats(const lapis_hip_csr_plan *plan, lapis_hip_csr_s
  *          so neighbouring lanes gather from the same 128-byte lines (fewer requests
  *          to L2, which is what bounds these matrices).  Row sums are LDS atomics
  *          shared by the wavefronts of the group: the order of additions, and with it
- *          the last bits of y, can differ between runs.  AUTO picks this one.
+ *          the last bits of y, can differ between runs.  Rows of 32768 entries or more
+ *          are left out of the copy and read from the crd/val passed to the SpMV call
+ *          (a second kernel).  Where several workgroups share a row block, and for the
+ *          long rows, y is updated with hardware floating-point atomics: y must be
+ *          ordinary (coarse-grained) device memory.  AUTO picks this layout.
  * The reference has no counterpart (its launch never looks at columns,
  * KokkosLoopMapping.cpp:861-862).  The copy holds the VALUES as they are now: build
  * again after changing val.  Selects the COLBLOCK kernel on success; SpMV calls with
- * this plan then ignore their crd/val arguments.  Synchronises `stream`. */
+ * this plan then read their crd/val arguments only for the long rows of the GROUP
+ * layout.  Synchronises `stream`. */
 enum lapis_hip_colblock_layout {
   LAPIS_HIP_COLBLOCK_AUTO = 0,
   LAPIS_HIP_COLBLOCK_WAVE = 1,
