@@ -116,10 +116,6 @@ def run_spmv(args, cfg):
     ms = elapsed / args.steps * 1e3
     family = "colgroup" if stats["colblock_layout_name"] == "group" else stats["kernel_name"]
     kernel_name = "spmv_%s_kernel<%s>" % (family, "double" if dtype == np.float64 else "float")
-    if family == "colgroup" and stats["max_row_len"] >= 32768:
-        # rows that long stay in CSR: the timed span runs from the start of the blocked
-        # kernel to the end of the long-row kernel behind it
-        kernel_name += " + spmv_long_piece_kernel"
     achieved = bytes_step / (kt["mean_ms"] * 1e-3) / 1e9
     out = {
         "metric": "CSR SpMV %s achieved HBM GB/s" % ("fp64" if dtype == np.float64 else "fp32"),

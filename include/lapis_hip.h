@@ -137,16 +137,17 @@ int lapis_hip_csr_plan_get_stats(const lapis_hip_csr_plan *plan, lapis_hip_csr_s
  *          so neighbouring lanes gather from the same 128-byte lines (fewer requests
  *          to L2, which is what bounds these matrices).  Row sums are LDS atomics
  *          shared by the wavefronts of the group: the order of additions, and with it
- *          the last bits of y, can differ between runs.  Rows of 32768 entries or more
- *          are left out of the copy and read from the crd/val passed to the SpMV call
- *          (a second kernel).  Where several workgroups share a row block, and for the
- *          long rows, y is updated with hardware floating-point atomics: y must be
- *          ordinary (coarse-grained) device memory.  AUTO picks this layout.
+ *          the last bits of y, can differ between runs.  Rows much longer than the
+ *          rest (>= max(1024, 16 x mean) entries) are numbered apart and fill row
+ *          blocks of their own; every block's entries are cut into equal work units,
+ *          one workgroup each, so skewed matrices balance.  Blocks cut into several
+ *          units, and the blocks of long rows, update y with hardware floating-point
+ *          atomics: y must be ordinary (coarse-grained) device memory.  AUTO picks
+ *          this layout.
  * The reference has no counterpart (its launch never looks at columns,
  * KokkosLoopMapping.cpp:861-862).  The copy holds the VALUES as they are now: build
  * again after changing val.  Selects the COLBLOCK kernel on success; SpMV calls with
- * this plan then read their crd/val arguments only for the long rows of the GROUP
- * layout.  Synchronises `stream`. */
+ * this plan then ignore their crd/val arguments.  Synchronises `stream`. */
 enum lapis_hip_colblock_layout {
   LAPIS_HIP_COLBLOCK_AUTO = 0,
   LAPIS_HIP_COLBLOCK_WAVE = 1,

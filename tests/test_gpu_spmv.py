@@ -119,25 +119,26 @@ def test_column_blocked_copy_matches_oracle(gpu, cases, slice_log2, layout):
         plan.destroy()
 
 
-@pytest.mark.parametrize("long_threshold,split,rows", [(64, 3, 4096), (1024, 1, 8192), (100000000, 7, 16384)])
-def test_workgroup_layout_with_forced_long_rows_and_splits(gpu, cases, monkeypatch, long_threshold, split, rows):
-    # the tuning overrides move rows between the blocked copy and the long-row pieces and
-    # change how many workgroups share a row block: every combination must give the same y
+@pytest.mark.parametrize("long_threshold,unit,rows", [(2, 100, 4096), (64, 5000, 4096), (1024, 0, 8192),
+                                                      (100000000, 33333, 16384)])
+def test_workgroup_layout_with_forced_long_rows_and_units(gpu, cases, monkeypatch, long_threshold, unit, rows):
+    # the tuning overrides move rows between their natural blocks and the blocks of long rows
+    # and change how many work units a block is cut into: every combination must give the same y
     monkeypatch.setenv("LAPIS_HIP_COLBLOCK_LONG", str(long_threshold))
-    monkeypatch.setenv("LAPIS_HIP_COLBLOCK_SPLIT", str(split))
+    monkeypatch.setenv("LAPIS_HIP_COLBLOCK_UNIT", str(unit))
     monkeypatch.setenv("LAPIS_HIP_COLBLOCK_ROWS", str(rows))
     dtype, built = cases
     for name, (A, x, y_in, want, scale) in built.items():
         if A.nnz == 0:
             continue
-        print("case", name, "group", long_threshold, split, rows, np.dtype(dtype).name, flush=True)
+        print("case", name, "group", long_threshold, unit, rows, np.dtype(dtype).name, flush=True)
         pos, crd, val = dev(A.pos), dev(A.crd), dev(A.val)
         plan = gpu.CsrPlan(A.nrows, A.ncols, pos, crd, value_bytes=np.dtype(dtype).itemsize)
         plan.build_colblock(crd, val, 7, layout="group")
         y = dev(y_in)
         gpu.spmv(plan, A.nrows, A.ncols, pos, crd, val, dev(x), y)
         torch.cuda.synchronize()
-        assert_rows_close(y.cpu().numpy(), want, scale, dtype, "%s/group long>=%d split %d" % (name, long_threshold, split))
+        assert_rows_close(y.cpu().numpy(), want, scale, dtype, "%s/group long>=%d unit %d" % (name, long_threshold, unit))
         plan.destroy()
 
 
