@@ -25,12 +25,13 @@ def _spmv_full(gpu, oracle, A, x, dtype):
     tdt = torch.float64 if dtype == np.float64 else torch.float32
     results = {}
     variants = [(0, 0, "auto"), (1, 0, "reference-width"), (2, 0, "rowblock"), (3, 0, "nnzsplit")]
+    variants.append((4, 0, "colblock-group"))
     if A.ncols <= (1 << 22):
-        variants.append((4, 0, "colblock"))
+        variants.append((4, 0, "colblock-wave"))
     for kid, width, name in variants:
         print("full-size", name, flush=True)
         if kid == 4:
-            plan.build_colblock(crd, val)
+            plan.build_colblock(crd, val, layout=name.split("-")[1])
         else:
             plan.set_kernel(kid, width)
         y = torch.zeros(A.nrows, dtype=tdt, device="cuda")

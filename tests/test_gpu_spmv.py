@@ -38,6 +38,9 @@ def _matrices(dtype):
     out["wide_gap_of_empty_rows"] = _from_lengths([7] * 10 + [0] * 1000 + [9] * 10, 64, 5, dtype)
     out["dense_short"] = _from_lengths([64] * 257, 64, 6, dtype)
     out["mean_100"] = gen.poisson_random(3000, 100.0, seed=7, dtype=dtype)
+    # rectangular: more columns than rows and the other way round
+    out["wide_300x100000"] = _from_lengths([40] * 150 + [3000] + [0] * 49 + [700] * 100, 100000, 8, dtype)
+    out["tall_50000x37"] = _from_lengths([5, 0, 37, 1] * 12500, 37, 9, dtype)
     return out
 
 
