@@ -46,8 +46,7 @@ struct lapis_hip_csr_plan {
 };
 
 namespace lapis {
-constexpr int kColblockRows = 1024;  // rows per wavefront in the column-blocked kernel
-constexpr int kColblockRowBits = 10;
+constexpr int kColblockRowBits = 10;  // the per-wavefront layout keeps up to 1024 rows per wavefront
 
 // bits needed for values 0..n-1
 inline int bits_for(int64_t n) {

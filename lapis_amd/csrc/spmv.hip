@@ -384,7 +384,6 @@ __global__ __launch_bounds__(256) void chunk_row_kernel(int nrows, int nchunks,
 using namespace lapis;
 
 namespace {
-constexpr int kChunk = 1024;      // non-zeros per wavefront in the row-split kernel
 constexpr int kRowblockCap = 1024;  // staged non-zeros per wavefront tile in the row-block kernel
 constexpr int kWavesPerBlock = 4;
 
