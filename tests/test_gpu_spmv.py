@@ -145,6 +145,42 @@ def test_workgroup_layout_with_forced_long_rows_and_units(gpu, cases, monkeypatc
         plan.destroy()
 
 
+def test_workgroup_layout_on_seeded_random_shapes(gpu, oracle, monkeypatch):
+    # 40 matrices of random shape, density and skew, each with its own slice width, work-unit size,
+    # long-row threshold and block size: unit borders fall inside tiles, on tile borders and
+    # next to empty tiles
+    rng = np.random.Generator(np.random.PCG64(20240607))
+    for case in range(40):
+        dtype = [np.float64, np.float32][case % 2]
+        nrows = int(rng.integers(1, 40000))
+        ncols = int(rng.integers(1, 300000))
+        mean = float(rng.choice([0.3, 2.0, 9.0, 40.0]))
+        lengths = np.minimum(rng.poisson(mean, nrows), ncols)
+        for _ in range(int(rng.integers(0, 4))):  # a few long rows
+            lengths[int(rng.integers(0, nrows))] = min(ncols, int(rng.integers(500, 60000)))
+        A = _from_lengths(lengths, ncols, 1000 + case, dtype)
+        if A.nnz == 0:
+            continue
+        slice_log2 = int(rng.integers(1, 19))
+        monkeypatch.setenv("LAPIS_HIP_COLBLOCK_UNIT", str(int(rng.choice([0, 64, 1000, 4096, 50000]))))
+        monkeypatch.setenv("LAPIS_HIP_COLBLOCK_LONG", str(int(rng.choice([0, 2, 300, 5000]))))
+        monkeypatch.setenv("LAPIS_HIP_COLBLOCK_ROWS", str(int(rng.choice([0, 4096, 8192, 16384]))))
+        x = gen.uniform_vector(A.ncols, 11, dtype=dtype)
+        y_in = gen.uniform_vector(A.nrows, 12, dtype=dtype)
+        want = y_in.copy()
+        oracle.spmv(A.pos, A.crd, A.val, x, want)
+        scale = oracle.spmv_abs_scale(A.pos, A.crd, A.val, x, y_in)
+        print("random case", case, nrows, ncols, A.nnz, int(lengths.max()), slice_log2, np.dtype(dtype).name, flush=True)
+        pos, crd, val = dev(A.pos), dev(A.crd), dev(A.val)
+        plan = gpu.CsrPlan(A.nrows, A.ncols, pos, crd, value_bytes=np.dtype(dtype).itemsize)
+        plan.build_colblock(crd, val, slice_log2, layout="group")
+        y = dev(y_in)
+        gpu.spmv(plan, A.nrows, A.ncols, pos, crd, val, dev(x), y)
+        torch.cuda.synchronize()
+        assert_rows_close(y.cpu().numpy(), want, scale, dtype, "random case %d" % case)
+        plan.destroy()
+
+
 def test_column_blocked_copy_refuses_what_it_cannot_encode(gpu):
     # per-wavefront layout: 2^23 columns need 23 bits; an entry has 22
     pos = dev(np.array([0, 1], np.int32))
