@@ -42,7 +42,10 @@ enum lapis_hip_status {
 int lapis_hip_init(void);
 /* Replaces `Kokkos::finalize()` of the emitted lapis_finalize() (emitter :4352-4376). */
 int lapis_hip_finalize(void);
-/* Message of the last non-OK status returned on the calling thread. */
+/* Message of the last non-OK status returned on the calling thread, and the name of
+ * a status code.  The reference has no status codes: its emitted code calls
+ * Kokkos::abort (LAPISSupport.hpp:76,86; emitter :1294-1301); the generated-module
+ * shim keeps that behaviour on top of these. */
 const char *lapis_hip_last_error(void);
 const char *lapis_hip_status_name(int status);
 /* Replaces Kokkos::DefaultExecutionSpace().fence() (emitter :2680-2682). */
@@ -121,6 +124,9 @@ int lapis_hip_csr_plan_create(lapis_hip_csr_plan **plan, int64_t nrows, int64_t 
 /* Overrides the automatic choice (tuning and tests).  `width` is used by SUBWARP
  * (0 = the reference's rule); other kernels ignore it. */
 int lapis_hip_csr_plan_set_kernel(lapis_hip_csr_plan *plan, int kernel, int width);
+/* The statistics and the choice, including what the reference's rule would have
+ * chosen (estimate of KokkosLoopMapping.cpp:279-323, vector length of
+ * LAPISSupport.hpp:428-435). */
 int lapis_hip_csr_plan_get_stats(const lapis_hip_csr_plan *plan, lapis_hip_csr_stats *stats);
 /* Opt-in layouts for matrices whose x does not fit the 4 MB L2 of an XCD (wide,
  * uniformly random columns).  crd/val are copied once into an order in which a
@@ -156,6 +162,8 @@ enum lapis_hip_colblock_layout {
 int lapis_hip_csr_plan_build_colblock(lapis_hip_csr_plan *plan, const int32_t *crd, const void *val,
                                       int value_bytes, int layout, int slice_log2_cols,
                                       lapis_hip_stream_t stream);
+/* Frees the plan's device buffers; emitted code would call it where lapis_finalize()
+ * frees the module's global views (emitter :4352-4376).  NULL is allowed. */
 int lapis_hip_csr_plan_destroy(lapis_hip_csr_plan *plan);
 
 /* ---- SpMV ------------------------------------------------------------------ */
