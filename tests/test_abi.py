@@ -80,3 +80,25 @@ def test_memref_descriptor_layout_is_stridedmemreftype():
 def test_specifier_flattening_matches_emitted_wrapper():
     flat = module._flatten_specifier(((5, 6), (6, 8, 8)))
     assert flat.dtype == np.int64 and list(flat) == [5, 6, 6, 8, 8]
+
+
+def test_missing_library_is_an_error_not_a_fallback(tmp_path):
+    with pytest.raises(FileNotFoundError, match="no CPU fallback"):
+        hip.load(str(tmp_path / "liblapis_hip.so"))
+    with pytest.raises(FileNotFoundError):
+        module.LAPISModule(str(tmp_path / "liblapis_package_module.so"))
+
+
+def test_nothing_under_the_package_reaches_for_the_oracle():
+    # the oracle is test infrastructure: the product must not import, load or run it
+    import os
+    import re
+    pkg = os.path.dirname(hip.__file__)
+    offenders = []
+    for root, _, files in os.walk(pkg):
+        for name in files:
+            if name.endswith((".py", ".hip", ".hpp", ".cpp", ".h")):
+                text = open(os.path.join(root, name), errors="ignore").read()
+                if re.search(r"liblapis_oracle|oracle\.oracle|from oracle|import oracle|lapis_oracle\.c", text):
+                    offenders.append(os.path.join(root, name))
+    assert offenders == []
