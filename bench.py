@@ -136,6 +136,28 @@ def run_spmv(args, cfg):
                      "traffic": traffic_from_profiles("%s_config%d" % (family, cfg)) if cfg else None,
                      "kernel_ms_mean": kt["mean_ms"], "kernel_ms_min": kt["min_ms"], "launches_timed": kt["count"]},
     }
+    if args.graph or cfg == 1:
+        # Launch-bound sizes: the same calls captured once into a HIP graph (10 per graph) and
+        # replayed, which takes the Python and launch overhead of each call out of the loop.
+        per_graph = 10
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            side.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                for _ in range(per_graph):
+                    hip.spmv(plan, A.nrows, A.ncols, pos, crd, val, dx, y)
+        torch.cuda.synchronize()
+        replays = max(1, args.steps // per_graph)
+        graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(replays):
+            graph.replay()
+        torch.cuda.synchronize()
+        gms = (time.perf_counter() - t0) / (replays * per_graph) * 1e3
+        out["graph_replay"] = {"calls_per_graph": per_graph, "ms_per_step": gms,
+                               "GB/s": bytes_step / (gms * 1e-3) / 1e9}
     if args.host_buffers:
         # The generated-module entry takes HOST arrays (the reference's Python path):
         # every call uploads the matrix and vectors and copies y back.  Reported beside
@@ -291,6 +313,8 @@ def main():
                     help="layout of the column-blocked copy (auto = group)")
     ap.add_argument("--width", type=int, default=0, help="lanes per row with --kernel subwarp (0 = the reference's rule)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--graph", action="store_true",
+                    help="also time the calls replayed from a HIP graph (always done for config 1)")
     ap.add_argument("--host-buffers", action="store_true",
                     help="also time the generated-module entry point, which takes host arrays (PCIe-inclusive)")
     ap.add_argument("--calibrate-copy", action="store_true",

@@ -290,3 +290,40 @@ def test_empty_matrix_is_a_no_op(gpu):
     y = torch.empty(0, dtype=torch.float64, device="cuda")
     gpu.spmv(plan, 0, 0, pos, crd, y, y, y)
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("kernel", ["rowblock", "nnzsplit", "colblock-group", "colblock-wave"])
+def test_spmv_replays_from_a_hip_graph(gpu, oracle, kernel):
+    # A planned SpMV is kernel launches only (no allocation, no host read, no memset), so a
+    # caller can capture it.  The graph is replayed several times with eager work and
+    # synchronisation in between, and every replay is checked against the eager result.
+    A, x = gen.config2(scale=1 / 64)
+    pos, crd, val, dx = dev(A.pos), dev(A.crd), dev(A.val), dev(x)
+    plan = gpu.CsrPlan(A.nrows, A.ncols, pos, crd)
+    if kernel.startswith("colblock"):
+        plan.build_colblock(crd, val, layout=kernel.split("-")[1])
+    else:
+        plan.set_kernel(KID[kernel], 0)
+    want = np.zeros(A.nrows)
+    oracle.spmv(A.pos, A.crd, A.val, x, want)
+    scale = oracle.spmv_abs_scale(A.pos, A.crd, A.val, x)
+    y = torch.zeros(A.nrows, dtype=torch.float64, device="cuda")
+    gpu.spmv(plan, A.nrows, A.ncols, pos, crd, val, dx, y)  # eager: also does the one-time kernel attribute call
+    torch.cuda.synchronize()
+    assert_rows_close(y.cpu().numpy(), want, scale, np.float64, kernel + " eager")
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        y.zero_()
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            gpu.spmv(plan, A.nrows, A.ncols, pos, crd, val, dx, y)
+    torch.cuda.synchronize()
+    for replay in range(3):
+        y.zero_()                       # eager work between the replays
+        scratch = (dx * 2.0).sum().item()  # and a host synchronisation
+        assert np.isfinite(scratch)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_rows_close(y.cpu().numpy(), want, scale, np.float64, "%s replay %d" % (kernel, replay))
+    plan.destroy()
