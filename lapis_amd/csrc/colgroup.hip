@@ -270,13 +270,13 @@ int launch_colgroup_threads(const lapis_hip_csr_plan *p, const T *x, T *y, hipSt
 template <typename T>
 int launch_colgroup(const lapis_hip_csr_plan *p, const T *x, T *y, hipStream_t st) {
   if (p->colblock_nunits == 0) return LAPIS_HIP_OK;
-  switch (p->colblock_rows) {
-    case 16384: return launch_colgroup_threads<T, 1024>(p, x, y, st);
-    case 8192: return launch_colgroup_threads<T, 512>(p, x, y, st);
-    case 4096: return launch_colgroup_threads<T, 256>(p, x, y, st);
+  switch (p->colblock_threads) {
+    case 1024: return launch_colgroup_threads<T, 1024>(p, x, y, st);
+    case 512: return launch_colgroup_threads<T, 512>(p, x, y, st);
+    case 256: return launch_colgroup_threads<T, 256>(p, x, y, st);
     default:
-      return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT, "colblock: no workgroup kernel for %d rows per block",
-                       p->colblock_rows);
+      return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT, "colblock: no workgroup kernel with %d threads",
+                       p->colblock_threads);
   }
 }
 template int launch_colgroup<double>(const lapis_hip_csr_plan *, const double *, double *, hipStream_t);
@@ -298,6 +298,21 @@ int build_colgroup(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int 
   if (rows != 4096 && rows != 8192 && rows != 16384) rows = nrows > 8192 ? 16384 : (nrows > 4096 ? 8192 : 4096);
   const int row_bits = bits_for(rows);
   slice_log2 = std::min(slice_log2, 32 - row_bits);  // an entry word holds row in block | column in slice
+  // Threads per workgroup: 16 rows per thread, but half of that where a tile holds about
+  // one or two entries per 128-byte line of x.  Such matrices are bound by requests to L2,
+  // and 8 wavefronts per CU, each with one gather in flight, measured 2-6 % faster than 16
+  // (4.2 M rows with 16 / 24 / 32 per row: 0.305 / 0.423 / 0.538 against 0.325 / 0.445 /
+  // 0.546 ms).  Dense tiles are bound by instruction issue and lose up to 40 % with half the
+  // threads (2.1 M rows, 32 per row: 0.265 against 0.248 ms; config 3: 0.225 against 0.161),
+  // and with a quarter of an entry per line the full workgroup is 2 % ahead again.
+  int threads = rows / 16;
+  {
+    const double per_line = (double)rows * p->stats.mean_row_len * (128.0 / sizeof(T)) /
+                            (double)std::max<int64_t>(1, p->stats.ncols);
+    if (rows == 16384 && per_line >= 0.5 && per_line < 2.5) threads = 512;
+    const int forced = env_or("LAPIS_HIP_COLBLOCK_THREADS", 0);
+    if (forced == 256 || forced == 512 || forced == 1024) threads = forced;
+  }
   const int nblocks_nat = (int)ceil_div(nrows, rows);
   // finer slices than LDS has room for tile pointers are widened (a matter of speed only)
   while (slice_log2 < 32 - row_bits && ceil_div(p->stats.ncols, 1LL << slice_log2) > kMaxSlicesInLds) ++slice_log2;
@@ -415,7 +430,7 @@ int build_colgroup(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int 
   // otherwise 1.25 x the mean block, so that only outsized blocks are cut.
   int64_t unit = env_or("LAPIS_HIP_COLBLOCK_UNIT", 0);
   if (unit <= 0) {
-    // workgroups of 16384 / 8192 / 4096 rows fit 1 / 2 / 4 to a CU (LDS and thread limits)
+    // workgroups of 16384 / 8192 / 4096 rows fit 1 / 2 / 4 to a CU (LDS limit)
     const int64_t cus = (int64_t)std::max(1, device_cu_count()) * (16384 / rows);
     int64_t nonempty = 0, longest = 1;
     for (int b = 0; b < nblocks; ++b) {
@@ -462,6 +477,7 @@ int build_colgroup(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int 
   p->colblock_group = 1;
   p->colblock_epl = env_or("LAPIS_HIP_COLBLOCK_EPL", 8);  // entries per thread and trip
   p->colblock_rows = rows;
+  p->colblock_threads = threads;
   p->colblock_nblocks = nblocks;
   p->colblock_nblocks_nat = nblocks_nat;
   p->colblock_nslices = nslices;

@@ -29,6 +29,7 @@ struct lapis_hip_csr_plan {
   int colblock_epl;          // entries per lane per step (1, 2 or 4)
   int colblock_pad;          // 1: workgroups of 8 wavefronts instead of 4
   int colblock_rows;         // rows per wavefront (512 or 1024), or per workgroup in the workgroup-blocked layout
+  int colblock_threads;      // threads per workgroup of the workgroup-blocked kernel (256, 512 or 1024)
   int colblock_group;        // 1: workgroup-blocked layout (tiles in column order, row sums shared by a workgroup)
   int colblock_nblocks;      // row blocks of the workgroup-blocked layout
   int colblock_nslices;      // slices of x
