@@ -110,3 +110,49 @@ def test_masked_cg_and_moments_match_oracle(gpu, oracle, golden):
     xo, ito, _ = oracle.pcg_masked(A.pos, A.crd, off, b * mk, mk, dd, 1e-9, 300)
     assert it == ito and it < 300
     assert np.allclose(x.cpu().numpy(), xo, rtol=1e-8, atol=1e-11)
+
+
+def test_iteration_counter_semantics_of_the_reference_loop(gpu, oracle):
+    # examples/pcg_solve.py:74-98: i starts at 1 and the loop leaves when !(relres > tol) or i == maxiter
+    A, b = gen.config5(scale=(12 / 192) ** 3)
+    one = np.ones(A.nrows)
+    for tol, maxiter in ((1e30, 50), (0.0, 1), (1e-3, 1000), (1e-6, 7)):
+        xo, io, ro = oracle.pcg(A.pos, A.crd, A.val, b, one, tol, maxiter)
+        xg, ig, rg = _solve(gpu, A.pos, A.crd, A.val, b, None, tol, maxiter)
+        assert ig == io, (tol, maxiter, ig, io)
+        assert np.allclose(xg, xo, rtol=1e-9, atol=1e-12)
+    # a huge tolerance leaves after the first pass, with one update applied
+    xg, ig, rg = _solve(gpu, A.pos, A.crd, A.val, b, None, 1e30, 50)
+    assert ig == 1 and np.any(xg != 0.0)
+
+
+def test_zero_right_hand_side_gives_nan_relres_and_one_pass(gpu, oracle):
+    # r0 = 0: relres = 0/0 is NaN, `relres > tol` is false, the loop leaves at i = 1 (reference semantics)
+    A, _ = gen.config5(scale=(10 / 192) ** 3)
+    b = np.zeros(A.nrows)
+    xo, io, ro = oracle.pcg(A.pos, A.crd, A.val, b, np.ones(A.nrows), 1e-10, 40)
+    xg, ig, rg = _solve(gpu, A.pos, A.crd, A.val, b, None, 1e-10, 40)
+    assert ig == io == 1
+    assert np.isnan(rg) == np.isnan(ro)
+
+
+def test_cg_with_a_column_blocked_plan(gpu, oracle):
+    # an SPD matrix with random columns: A = B + B^T + diagonal shift, solved with the
+    # workgroup-blocked SpMV inside the CG driver
+    import scipy.sparse as sp
+    R = gen.poisson_random(20000, 6.0, seed=5)
+    B = sp.csr_matrix((np.abs(R.val), R.crd, R.pos), shape=(R.nrows, R.ncols))
+    S = (B + B.T).tocsr()
+    S = (S + sp.diags(np.asarray(S.sum(axis=1)).ravel() + 1.0)).tocsr()
+    S.sort_indices()
+    pos, crd, val = S.indptr.astype(np.int32), S.indices.astype(np.int32), S.data.astype(np.float64)
+    n = S.shape[0]
+    b = S @ np.ones(n)
+    xo, io, ro = oracle.pcg(pos, crd, val, b, np.ones(n), 1e-10, 200)
+    dpos, dcrd, dval = dev(pos), dev(crd), dev(val)
+    plan = gpu.CsrPlan(n, n, dpos, dcrd)
+    plan.build_colblock(dcrd, dval, 8, layout="group")
+    x = torch.zeros(n, dtype=torch.float64, device="cuda")
+    ig, rg = gpu.pcg(plan, n, dpos, dcrd, dval, dev(b), None, 1e-10, 200, x)
+    assert rg <= 1e-10 and abs(ig - io) <= 1  # the sums are added in another order: the count may move by one
+    assert np.allclose(x.cpu().numpy(), np.ones(n), rtol=1e-8, atol=1e-8)
