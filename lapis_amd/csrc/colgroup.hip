@@ -298,18 +298,19 @@ int build_colgroup(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int 
   if (rows != 4096 && rows != 8192 && rows != 16384) rows = nrows > 8192 ? 16384 : (nrows > 4096 ? 8192 : 4096);
   const int row_bits = bits_for(rows);
   slice_log2 = std::min(slice_log2, 32 - row_bits);  // an entry word holds row in block | column in slice
-  // Threads per workgroup: 16 rows per thread, but half of that where a tile holds about
-  // one or two entries per 128-byte line of x.  Such matrices are bound by requests to L2,
+  // Threads per workgroup: 16 rows per thread, but half of that where a tile holds at most
+  // about two entries per 128-byte line of x.  Such matrices are bound by requests to L2,
   // and 8 wavefronts per CU, each with one gather in flight, measured 2-6 % faster than 16
   // (4.2 M rows with 16 / 24 / 32 per row: 0.305 / 0.423 / 0.538 against 0.325 / 0.445 /
   // 0.546 ms).  Dense tiles are bound by instruction issue and lose up to 40 % with half the
-  // threads (2.1 M rows, 32 per row: 0.265 against 0.248 ms; config 3: 0.225 against 0.161),
-  // and with a quarter of an entry per line the full workgroup is 2 % ahead again.
+  // threads (2.1 M rows, 32 per row: 0.265 against 0.248 ms; config 3: 0.225 against 0.161).
+  // With a quarter of an entry per line it is 0.123 against 0.129 ms (4.2 M rows, 4 per row)
+  // but 0.519 against 0.509 ms when the blocks need two rounds (8.4 M rows, 8 per row).
   int threads = rows / 16;
   {
     const double per_line = (double)rows * p->stats.mean_row_len * (128.0 / sizeof(T)) /
                             (double)std::max<int64_t>(1, p->stats.ncols);
-    if (rows == 16384 && per_line >= 0.5 && per_line < 2.5) threads = 512;
+    if (rows == 16384 && per_line < 2.5) threads = 512;
     const int forced = env_or("LAPIS_HIP_COLBLOCK_THREADS", 0);
     if (forced == 256 || forced == 512 || forced == 1024) threads = forced;
   }
