@@ -327,3 +327,27 @@ def test_spmv_replays_from_a_hip_graph(gpu, oracle, kernel):
         torch.cuda.synchronize()
         assert_rows_close(y.cpu().numpy(), want, scale, np.float64, "%s replay %d" % (kernel, replay))
     plan.destroy()
+
+
+def test_plans_give_back_their_device_memory(gpu):
+    # build and destroy plans with both column-blocked layouts (long rows included) many times:
+    # the free device memory must come back to where it was
+    A = gen.powerlaw_random(131072, 30.0, 200000, seed=3003, dtype=np.float64)
+    pos, crd, val = dev(A.pos), dev(A.crd), dev(A.val)
+    torch.cuda.synchronize()
+
+    def cycle():
+        for layout in ("group", "wave", "group"):
+            plan = gpu.CsrPlan(A.nrows, A.ncols, pos, crd)
+            plan.build_colblock(crd, val, 0, layout=layout)
+            plan.build_colblock(crd, val, 9, layout="group")  # rebuilding replaces the copy
+            plan.destroy()
+
+    cycle()  # first use may grow library-internal pools (radix sort, kernel code)
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    for _ in range(5):
+        cycle()
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free0 - free1 < (8 << 20), "plans leak %.1f MB over 15 build/destroy cycles" % ((free0 - free1) / 1e6)
