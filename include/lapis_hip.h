@@ -213,6 +213,18 @@ int lapis_hip_dot_f64(int64_t n, const double *x, const double *y, double init, 
                       lapis_hip_stream_t stream);
 int lapis_hip_dot_f32(int64_t n, const float *x, const float *y, float init, float *result,
                       lapis_hip_stream_t stream);
+/* lapis_hip_dot_f64 for callers that cannot allocate (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same kernels and the same result, bit for bit, as lapis_hip_dot_f64, but
+ * the block partials live in a fixed 16 KB array inside the library's code object
+ * (one copy per GPU, held until the process ends) instead of an allocated ring: the
+ * call performs no hipMalloc / hipFree.  n above LAPIS_HIP_DOT_NOALLOC_MAX_N is
+ * rejected with LAPIS_HIP_ERR_INVALID_ARGUMENT.  All calls on one GPU share the one
+ * array: calls that overlap on one GPU (different streams or threads) race; order
+ * them on one stream. */
+#define LAPIS_HIP_DOT_NOALLOC_MAX_N (INT64_C(1) << 34)
+int lapis_hip_dot_f64_noalloc(int64_t n, const double *x, const double *y, double init, double *result,
+                              lapis_hip_stream_t stream);
 /* dst[i] = a*x[i] + b*y[i] (examples/pcg_solve.py:30-38; RangePolicy parallel_for,
  * emitter :1710-1715).  dst may alias x or y. */
 int lapis_hip_axpby_f64(int64_t n, double a, const double *x, double b, const double *y, double *dst,

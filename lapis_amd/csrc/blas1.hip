@@ -182,6 +182,30 @@ int take_slot(void **partials) {
   return LAPIS_HIP_OK;
 }
 
+// ---- the dot that allocates nothing ------------------------------------------------
+// Partials of lapis_hip_dot_f64_noalloc: a fixed array in the code object instead of the
+// ring above, so the entry point never calls hipMalloc.  Every GPU holds its own copy at
+// its own address; host code uses the address hipGetSymbolAddress returns for the
+// current device, never the array's name.
+static __device__ __align__(256) double g_dot_noalloc_scratch[kDotMaxBlocks];
+constexpr int kMaxDevices = 64;
+std::mutex g_noalloc_mutex;
+double *g_noalloc_ptr[kMaxDevices] = {};
+
+int noalloc_scratch(double **out) {
+  int dev = 0;
+  LAPIS_HIP_TRY(hipGetDevice(&dev));
+  LAPIS_REQUIRE(dev >= 0 && dev < kMaxDevices, "dot_f64_noalloc: device ordinal %d outside [0, %d)", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_noalloc_mutex);
+  if (!g_noalloc_ptr[dev]) {
+    void *p = nullptr;
+    LAPIS_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(g_dot_noalloc_scratch)));
+    g_noalloc_ptr[dev] = static_cast<double *>(p);
+  }
+  *out = g_noalloc_ptr[dev];
+  return LAPIS_HIP_OK;
+}
+
 template <typename T>
 int dot_entry(const char *what, int64_t n, const T *x, const T *y, T init, T *result, lapis_hip_stream_t stream) {
   LAPIS_CHECK_INIT();
@@ -195,9 +219,41 @@ int dot_entry(const char *what, int64_t n, const T *x, const T *y, T init, T *re
 }
 }  // namespace
 
+// Resolves the no-alloc scratch of the current device (called by lapis_hip_init, so that
+// the first lapis_hip_dot_f64_noalloc call does no set-up work either).
+int dot_noalloc_setup() {
+  double *p = nullptr;
+  return noalloc_scratch(&p);
+}
+
+// Gives the ring of partials back (lapis_hip_finalize at reference count zero).
+void dot_release_scratch() {
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch) (void)hipFree(g_scratch);
+  g_scratch = nullptr;
+  g_next_slot = 0;
+}
+
 }  // namespace lapis
 
 using namespace lapis;
+
+extern "C" int lapis_hip_dot_f64_noalloc(int64_t n, const double *x, const double *y, double init, double *result,
+                                         lapis_hip_stream_t stream) {
+  LAPIS_CHECK_INIT();
+  LAPIS_REQUIRE(n >= 0, "dot_f64_noalloc: negative length");
+  if (n > LAPIS_HIP_DOT_NOALLOC_MAX_N)
+    return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT, "dot_f64_noalloc: n=%lld exceeds the maximum of %lld elements",
+                     (long long)n, (long long)LAPIS_HIP_DOT_NOALLOC_MAX_N);
+  LAPIS_REQUIRE(result, "dot_f64_noalloc: null result");
+  LAPIS_REQUIRE(n == 0 || (x && y), "dot_f64_noalloc: null vector with n=%lld", (long long)n);
+  double *partials = nullptr;
+  const int rc = noalloc_scratch(&partials);
+  if (rc != LAPIS_HIP_OK) return rc;
+  // dot_partial_kernel writes every partial the final kernel reads (dot_grid(n) of them):
+  // nothing of the previous call's contents is read, so nothing has to be cleared.
+  return launch_dot<double>(n, x, y, init, result, partials, as_stream(stream));
+}
 
 extern "C" int lapis_hip_dot_f64(int64_t n, const double *x, const double *y, double init, double *result,
                                  lapis_hip_stream_t stream) {

@@ -15,4 +15,9 @@ int dot_grid(int64_t n);
 template <typename T>
 int launch_dot(int64_t n, const T *x, const T *y, T init, T *result, T *partials, hipStream_t st);
 
+// Per-device set-up of lapis_hip_dot_f64_noalloc (address of its fixed scratch array) and
+// release of the allocated ring of partials the other dot entry points use.
+int dot_noalloc_setup();
+void dot_release_scratch();
+
 }  // namespace lapis

@@ -4,6 +4,7 @@
 #include <mutex>
 #include <vector>
 
+#include "blas1.hpp"
 #include "common.hpp"
 
 namespace lapis {
@@ -69,6 +70,8 @@ extern "C" int lapis_hip_init(void) {
     return set_error(LAPIS_HIP_ERR_UNSUPPORTED_DEVICE, "lapis_hip_init: wavefront size %d, expected 64",
                      prop.warpSize);
   g_cu_count = prop.multiProcessorCount;
+  const int rc = dot_noalloc_setup();
+  if (rc != LAPIS_HIP_OK) return rc;
   g_refcount = 1;
   return LAPIS_HIP_OK;
 }
@@ -77,7 +80,7 @@ extern "C" int lapis_hip_finalize(void) {
   std::lock_guard<std::mutex> lock(g_mutex);
   if (g_refcount <= 0)
     return set_error(LAPIS_HIP_ERR_NOT_INITIALIZED, "lapis_hip_finalize: not initialized");
-  --g_refcount;
+  if (--g_refcount == 0) dot_release_scratch();
   return LAPIS_HIP_OK;
 }
 

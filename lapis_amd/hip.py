@@ -60,6 +60,7 @@ _SIGNATURES = {
     "lapis_hip_bspmm_csrv_f32_i32": [_i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp],
     "lapis_hip_dot_f64": [_i64, _vp, _vp, _dbl, _vp, _vp],
     "lapis_hip_dot_f32": [_i64, _vp, _vp, _flt, _vp, _vp],
+    "lapis_hip_dot_f64_noalloc": [_i64, _vp, _vp, _dbl, _vp, _vp],
     "lapis_hip_axpby_f64": [_i64, _dbl, _vp, _dbl, _vp, _vp, _vp],
     "lapis_hip_axpby_f32": [_i64, _flt, _vp, _flt, _vp, _vp, _vp],
     "lapis_hip_mult_f64": [_i64, _vp, _vp, _vp, _vp],
@@ -232,6 +233,13 @@ def dot(x, y, result, init_value=0.0, stream=None):
     lib = init()
     fn = getattr(lib, "lapis_hip_dot_%s" % _suffix(x))
     check(fn(int(x.shape[0]), _ptr(x), _ptr(y), init_value, _ptr(result), _stream(stream)))
+    return result
+
+
+def dot_noalloc(x, y, result, init_value=0.0, stream=None):
+    """dot() through the entry point that allocates nothing (fp64; fixed scratch inside the library)."""
+    lib = init()
+    check(lib.lapis_hip_dot_f64_noalloc(int(x.shape[0]), _ptr(x), _ptr(y), init_value, _ptr(result), _stream(stream)))
     return result
 
 
