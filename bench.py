@@ -31,13 +31,21 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def traffic_from_profiles(kernel_key):
-    """HBM bytes per launch measured with rocprofv3 --pmc (profiles/traffic.json), or None."""
+def traffic_from_profiles(kernel_key, kernel_ms):
+    """HBM bytes per launch measured with rocprofv3 --pmc (profiles/traffic.json), or None.
+
+    The figure belongs to the kernel as it was when it was profiled: it is given only when this run's
+    mean kernel time is within 20 % of the time recorded beside it, otherwise None (stale or unprofiled)."""
     path = os.path.join(ROOT, "profiles", "traffic.json")
     if not os.path.exists(path):
         return None
     with open(path) as f:
-        return json.load(f).get(kernel_key, {}).get("hbm_bytes_per_launch")
+        entry = json.load(f).get(kernel_key)
+    if not entry or not entry.get("kernel_ms_at_profile"):
+        return None
+    if abs(kernel_ms - entry["kernel_ms_at_profile"]) > 0.2 * entry["kernel_ms_at_profile"]:
+        return None
+    return entry["hbm_bytes_per_launch"]
 
 
 def cpu_baseline_spmv(A, x, budget_s=12.0):
@@ -94,13 +102,33 @@ def run_spmv(args, cfg):
     torch.cuda.synchronize()
     plan_ms = (time.perf_counter() - t0) * 1e3
     build_ms = None
-    if args.kernel == "colblock" or (args.kernel is None and plan.stats()["colblock_recommended"]):
+    csr_ms = None
+    if args.kernel == "colblock":
         t0 = time.perf_counter()
         plan.build_colblock(crd, val, layout=args.colblock_layout)
         torch.cuda.synchronize()
         build_ms = (time.perf_counter() - t0) * 1e3
     elif args.kernel:
         plan.set_kernel({"subwarp": 1, "rowblock": 2, "nnzsplit": 3}[args.kernel], args.width)
+    else:
+        # The library decides (lapis_hip_csr_plan_analyze): it builds the column-blocked copy where the
+        # row/column statistics call for it.  The CSR kernel the plan would otherwise launch is timed first,
+        # so that the number of calls after which the copy has paid for itself can be stated.
+        for _ in range(3):
+            hip.spmv(plan, A.nrows, A.ncols, pos, crd, val, dx, y)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(10):
+            hip.spmv(plan, A.nrows, A.ncols, pos, crd, val, dx, y)
+        torch.cuda.synchronize()
+        csr_ms = (time.perf_counter() - t0) / 10 * 1e3
+        y.zero_()
+        before = plan.stats()["kernel_name"]
+        t0 = time.perf_counter()
+        plan.analyze(crd, val)
+        torch.cuda.synchronize()
+        if plan.stats()["kernel_name"] != before:
+            build_ms = (time.perf_counter() - t0) * 1e3
     stats = plan.stats()
     for _ in range(args.warmup):
         hip.spmv(plan, A.nrows, A.ncols, pos, crd, val, dx, y)
@@ -128,12 +156,15 @@ def run_spmv(args, cfg):
                    "algorithmic_bytes_per_step": bytes_step, "kernel": stats["kernel_name"],
                    "colblock_layout": stats["colblock_layout_name"],
                    "width": stats["width"], "chunk": stats["chunk"],
-                   "reference_vector_length": stats["reference_vector_length"], "plan_ms": plan_ms},
+                   "reference_vector_length": stats["reference_vector_length"], "plan_ms": plan_ms,
+                   "csr_kernel_ms_per_call": csr_ms,
+                   # calls of this matrix after which building the copy (outside the timed region) has paid back
+                   "break_even_calls": (build_ms / (csr_ms - ms) if build_ms and csr_ms and csr_ms > ms else None)},
         "pct_of_hbm_peak": 100.0 * bytes_step / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "gflops": 2.0 * A.nnz / (ms * 1e-3) / 1e9,
         "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": traffic_from_profiles("%s_config%d" % (family, cfg)) if cfg else None,
+                     "traffic": traffic_from_profiles("%s_config%d" % (family, cfg), kt["mean_ms"]) if cfg else None,
                      "kernel_ms_mean": kt["mean_ms"], "kernel_ms_min": kt["min_ms"], "launches_timed": kt["count"]},
     }
     if args.graph or cfg == 1:
@@ -223,7 +254,7 @@ def run_spmm(args):
         "gflops": 2.0 * A.nnz * k / (ms * 1e-3) / 1e9,
         "roofline": {"bound": "hbm", "kernel": "spmm_wave_row_kernel<float,16>", "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": traffic_from_profiles("spmm_config4"), "kernel_ms_mean": kt["mean_ms"],
+                     "traffic": traffic_from_profiles("spmm_config4", kt["mean_ms"]), "kernel_ms_mean": kt["mean_ms"],
                      "launches_timed": kt["count"]},
     }
     if not args.no_cpu:
@@ -276,7 +307,7 @@ def run_cg(args):
         "gflops": (2.0 * A.nnz + 2 * 2 * n + 3 * 3 * n) / (ms * 1e-3) / 1e9,
         "roofline": {"bound": "hbm", "kernel": "spmv_%s_kernel<double>" % plan.stats()["kernel_name"],
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": traffic_from_profiles("cg_spmv_config5"), "kernel_ms_mean": kt["mean_ms"],
+                     "traffic": traffic_from_profiles("cg_spmv_config5", kt["mean_ms"]), "kernel_ms_mean": kt["mean_ms"],
                      "launches_timed": kt["count"]},
     }
     if not args.no_cpu:

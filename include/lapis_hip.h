@@ -99,10 +99,10 @@ typedef struct lapis_hip_csr_stats {
   int32_t kernel;      /* enum lapis_hip_spmv_kernel, never AUTO */
   int32_t width;       /* lanes per row for SUBWARP, else 0 */
   int32_t chunk;       /* non-zeros per wavefront for NNZSPLIT (512, 1024 or 2048), else 0 */
-  /* 1 if lapis_hip_csr_plan_build_colblock is expected to pay for this matrix (the
-   * gathers of a 1024-non-zero chunk range over more of x than an XCD's L2 keeps, and
-   * the matrix has at least 2^20 non-zeros); plan creation cannot build the copy
-   * itself because it is not given the values */
+  /* 1 if the column-blocked copy is expected to pay for this matrix (the gathers of a
+   * 1024-non-zero chunk range over more of x than an XCD's L2 keeps, and the matrix has
+   * at least 2^20 non-zeros); lapis_hip_csr_plan_analyze builds it when this is set
+   * (plan creation cannot: it is not given the values) */
   int32_t colblock_recommended;
   /* enum lapis_hip_colblock_layout of the copy this plan holds, 0 if none */
   int32_t colblock_layout;
@@ -121,6 +121,25 @@ typedef struct lapis_hip_csr_plan lapis_hip_csr_plan;
 int lapis_hip_csr_plan_create(lapis_hip_csr_plan **plan, int64_t nrows, int64_t ncols, int64_t nnz,
                               const int32_t *pos, const int32_t *crd, int value_bytes,
                               lapis_hip_stream_t stream);
+/* Second half of the loop-mapping decision, for callers that will run many SpMVs with
+ * one matrix: given the values too, builds the column-blocked copy
+ * (lapis_hip_csr_plan_build_colblock, AUTO layout) when the statistics recommend it, and
+ * selects that kernel; otherwise leaves the plan as it is.  The copy costs about as
+ * much as 40 SpMVs of the same matrix (one radix sort).  If the plan already holds a
+ * copy made from `crd`, only its values are refreshed.  No counterpart in the reference
+ * (its launch never looks at columns, KokkosLoopMapping.cpp:861-862).  Synchronises
+ * `stream`. */
+int lapis_hip_csr_plan_analyze(lapis_hip_csr_plan *plan, const int32_t *crd, const void *val, int value_bytes,
+                               lapis_hip_stream_t stream);
+/* Brings the values of the plan's column-blocked copy up to date with `val` (the
+ * caller's CSR values, same order as at build time): one gather pass through the kept
+ * sort permutation, no sort, no synchronisation.  The reference reads val on every
+ * call (tests/Dialect/Kokkos/loop_mapping_2.mlir.gold:22); a copy cannot, so callers
+ * that change values in place call this afterwards.  `val` may be a different buffer
+ * than before: later SpMV calls must then pass this one.  A plan without a copy is left
+ * alone (status OK). */
+int lapis_hip_csr_plan_update_values(lapis_hip_csr_plan *plan, const void *val, int value_bytes,
+                                     lapis_hip_stream_t stream);
 /* Overrides the automatic choice (tuning and tests).  `width` is used by SUBWARP
  * (0 = the reference's rule); other kernels ignore it. */
 int lapis_hip_csr_plan_set_kernel(lapis_hip_csr_plan *plan, int kernel, int width);
@@ -144,16 +163,18 @@ int lapis_hip_csr_plan_get_stats(const lapis_hip_csr_plan *plan, lapis_hip_csr_s
  *          to L2, which is what bounds these matrices).  Row sums are LDS atomics
  *          shared by the wavefronts of the group: the order of additions, and with it
  *          the last bits of y, can differ between runs.  Rows much longer than the
- *          rest (>= max(1024, 16 x mean) entries) are numbered apart and fill row
+ *          rest (>= max(2048, 16 x mean) entries) are numbered apart and fill row
  *          blocks of their own; every block's entries are cut into equal work units,
  *          one workgroup each, so skewed matrices balance.  Blocks cut into several
  *          units, and the blocks of long rows, update y with hardware floating-point
  *          atomics: y must be ordinary (coarse-grained) device memory.  AUTO picks
  *          this layout.
  * The reference has no counterpart (its launch never looks at columns,
- * KokkosLoopMapping.cpp:861-862).  The copy holds the VALUES as they are now: build
- * again after changing val.  Selects the COLBLOCK kernel on success; SpMV calls with
- * this plan then ignore their crd/val arguments.  Synchronises `stream`. */
+ * KokkosLoopMapping.cpp:861-862).  The copy holds the VALUES as they are now: after
+ * changing val call lapis_hip_csr_plan_update_values (the sort permutation is kept,
+ * 4 bytes per non-zero).  Selects the COLBLOCK kernel on success; SpMV calls with this
+ * plan must pass the same crd and val buffers the copy was made from, anything else is
+ * refused with LAPIS_HIP_ERR_PLAN_MISMATCH.  Synchronises `stream`. */
 enum lapis_hip_colblock_layout {
   LAPIS_HIP_COLBLOCK_AUTO = 0,
   LAPIS_HIP_COLBLOCK_WAVE = 1,
@@ -254,7 +275,8 @@ int lapis_hip_scale_f64(int64_t n, double alpha, double *val, lapis_hip_stream_t
  * inside).  Scalars stay on the device between kernels; the host looks at the
  * convergence flag every few iterations only.  `iters` and `relres` are HOST
  * outputs; the call synchronises `stream` before returning.
- * `plan` may be NULL (one is built and destroyed inside). */
+ * `plan` may be NULL (one is built and destroyed inside, with the column-blocked copy
+ * when the matrix calls for it and maxiter >= 64 lets it pay back). */
 int lapis_hip_pcg_f64_i32(lapis_hip_csr_plan *plan, int64_t n, const int32_t *pos, const int32_t *crd,
                           const double *val, const double *b, const double *dinv, double tol,
                           uint64_t maxiter, double *x, uint64_t *iters, double *relres, double *work,
@@ -270,7 +292,8 @@ int lapis_hip_pcg_masked_f64_i32(lapis_hip_csr_plan *plan, int64_t n, const int3
 
 /* func @mht of examples/hitting_times.py:153-179: scales val by alpha IN PLACE
  * (scale_csr, :51-71), then two masked CG solves for the first two hitting-time
- * moments.  Synchronises `stream`. */
+ * moments.  A column-blocked copy in `plan` is refreshed after the scaling.
+ * Synchronises `stream`. */
 int lapis_hip_mht_f64_i32(lapis_hip_csr_plan *plan, int64_t n, int64_t nnz, const int32_t *pos,
                           const int32_t *crd, double *val, const double *mask, const double *d, double alpha,
                           double tol, uint64_t maxiter, double *mom1, double *mom2, lapis_hip_stream_t stream);

@@ -334,6 +334,9 @@ int pcg_run(lapis_hip_csr_plan *plan, int64_t n, const int32_t *pos, const int32
     PCG_TRY(hipStreamSynchronize(st));
     PCG_RC(lapis_hip_csr_plan_create(&own_plan, n, n, nnz32, pos, crd, 8, stream));
     plan = own_plan;
+    // the column-blocked copy costs about as much as 40 SpMVs of such a matrix: build it
+    // only when the iteration limit allows it to pay back
+    if (maxiter >= 64) PCG_RC(lapis_hip_csr_plan_analyze(own_plan, crd, val, 8, stream));
   }
   if (!work) {
     // own scratch: an even stride keeps all four vectors 16-byte aligned
@@ -451,6 +454,8 @@ extern "C" int lapis_hip_mht_f64_i32(lapis_hip_csr_plan *plan, int64_t n, int64_
   uint64_t its = 0;
   double res = 0.0;
   int rc = lapis_hip_scale_f64(nnz, alpha, val, stream);  // scale_csr, in place
+  // a column-blocked copy inside the caller's plan still holds the unscaled values
+  if (rc == LAPIS_HIP_OK && plan) rc = lapis_hip_csr_plan_update_values(plan, val, 8, stream);
   if (rc == LAPIS_HIP_OK) rc = lapis_hip_mult_f64(n, d, mask, bbuf, stream);
   if (rc == LAPIS_HIP_OK)
     rc = lapis_hip_pcg_masked_f64_i32(plan, n, pos, crd, val, bbuf, mask, d, tol, maxiter, mom1, &its, &res, nullptr,

@@ -196,9 +196,71 @@ __global__ __launch_bounds__(256) void colblock_low_word_kernel(long long n, con
 }
 
 
+namespace {
+__global__ __launch_bounds__(256) void iota_kernel(long long n, unsigned *__restrict__ out) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) out[i] = (unsigned)i;
+}
+template <typename T>
+__global__ __launch_bounds__(256) void gather_values_kernel(long long n, const unsigned *__restrict__ perm,
+                                                            const T *__restrict__ val, T *__restrict__ out) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) out[i] = val[perm[i]];
+}
+}  // namespace
+
+int sort_keys_with_perm(const unsigned long long *keys_in, int64_t nnz, int end_bit, unsigned long long **keys_out,
+                        unsigned **perm, hipStream_t st) {
+  unsigned *iota = nullptr;
+  void *temp = nullptr;
+  size_t temp_bytes = 0;
+  *keys_out = nullptr;
+  *perm = nullptr;
+  auto fail = [&](hipError_t e, const char *what) {
+    if (iota) (void)hipFree(iota);
+    if (temp) (void)hipFree(temp);
+    if (*keys_out) (void)hipFree(*keys_out);
+    if (*perm) (void)hipFree(*perm);
+    *keys_out = nullptr;
+    *perm = nullptr;
+    return set_error(LAPIS_HIP_ERR_RUNTIME, "csr_plan_build_colblock: %s failed: %s", what, hipGetErrorString(e));
+  };
+  hipError_t e;
+  if ((e = hipMalloc(&iota, sizeof(unsigned) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
+  if ((e = hipMalloc(keys_out, sizeof(unsigned long long) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
+  if ((e = hipMalloc(perm, sizeof(unsigned) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
+  hipLaunchKernelGGL(iota_kernel, dim3((unsigned)ceil_div(nnz, 256)), dim3(256), 0, st, (long long)nnz, iota);
+  if ((e = hipGetLastError()) != hipSuccess) return fail(e, "index kernel");
+  if ((e = hipcub::DeviceRadixSort::SortPairs(nullptr, temp_bytes, keys_in, *keys_out, iota, *perm, (int)nnz, 0, end_bit,
+                                              st)) != hipSuccess)
+    return fail(e, "radix sort sizing");
+  if ((e = hipMalloc(&temp, temp_bytes ? temp_bytes : 1)) != hipSuccess) return fail(e, "hipMalloc");
+  if ((e = hipcub::DeviceRadixSort::SortPairs(temp, temp_bytes, keys_in, *keys_out, iota, *perm, (int)nnz, 0, end_bit,
+                                              st)) != hipSuccess)
+    return fail(e, "radix sort");
+  if ((e = hipStreamSynchronize(st)) != hipSuccess) return fail(e, "synchronize");
+  (void)hipFree(iota);
+  (void)hipFree(temp);
+  return LAPIS_HIP_OK;
+}
+
+template <typename T>
+int gather_values(const unsigned *perm, const T *val, T *out, int64_t nnz, hipStream_t st) {
+  if (nnz == 0) return LAPIS_HIP_OK;
+  hipLaunchKernelGGL((gather_values_kernel<T>), dim3((unsigned)ceil_div(nnz, 256)), dim3(256), 0, st, (long long)nnz,
+                     perm, val, out);
+  LAPIS_LAUNCH_CHECK();
+  return LAPIS_HIP_OK;
+}
+template int gather_values<double>(const unsigned *, const double *, double *, int64_t, hipStream_t);
+template int gather_values<float>(const unsigned *, const float *, float *, int64_t, hipStream_t);
+
 void free_colblock(lapis_hip_csr_plan *p) {
   if (p->colblock_idx) (void)hipFree(p->colblock_idx);
   if (p->colblock_val) (void)hipFree(p->colblock_val);
+  if (p->colblock_perm) (void)hipFree(p->colblock_perm);
+  p->colblock_perm = nullptr;
+  p->colblock_src_crd = p->colblock_src_val = nullptr;
   if (p->colblock_tile_ptr) (void)hipFree(p->colblock_tile_ptr);
   if (p->colblock_units) (void)hipFree(p->colblock_units);
   if (p->colblock_long_rows) (void)hipFree(p->colblock_long_rows);
@@ -352,42 +414,44 @@ int build(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int slice_log
 
   unsigned long long *keys_in = nullptr, *keys_out = nullptr;
   T *val_out = nullptr;
-  unsigned *idx = nullptr;
-  void *temp = nullptr;
-  size_t temp_bytes = 0;
+  unsigned *idx = nullptr, *perm = nullptr;
   auto fail = [&](hipError_t e, const char *what) {
     if (keys_in) (void)hipFree(keys_in);
     if (keys_out) (void)hipFree(keys_out);
     if (val_out) (void)hipFree(val_out);
     if (idx) (void)hipFree(idx);
-    if (temp) (void)hipFree(temp);
+    if (perm) (void)hipFree(perm);
     return set_error(LAPIS_HIP_ERR_RUNTIME, "csr_plan_build_colblock: %s failed: %s", what, hipGetErrorString(e));
   };
   hipError_t e;
   if ((e = hipMalloc(&keys_in, sizeof(unsigned long long) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
-  if ((e = hipMalloc(&keys_out, sizeof(unsigned long long) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
   if ((e = hipMalloc(&val_out, sizeof(T) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
   if ((e = hipMalloc(&idx, sizeof(unsigned) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
   hipLaunchKernelGGL(colblock_keys_kernel, dim3((unsigned)ceil_div(nrows, 4)), dim3(256), 0, st, (int)nrows,
                      p->colblock_rows, col_bits,
                      slice_log2, slice_bits, p->pos, crd, keys_in);
   if ((e = hipGetLastError()) != hipSuccess) return fail(e, "key kernel");
-  if ((e = hipcub::DeviceRadixSort::SortPairs(nullptr, temp_bytes, keys_in, keys_out, val, val_out, (int)nnz, 0,
-                                              end_bit, st)) != hipSuccess)
-    return fail(e, "radix sort sizing");
-  if ((e = hipMalloc(&temp, temp_bytes ? temp_bytes : 1)) != hipSuccess) return fail(e, "hipMalloc");
-  if ((e = hipcub::DeviceRadixSort::SortPairs(temp, temp_bytes, keys_in, keys_out, val, val_out, (int)nnz, 0, end_bit,
-                                              st)) != hipSuccess)
-    return fail(e, "radix sort");
+  {
+    const int rc = sort_keys_with_perm(keys_in, nnz, end_bit, &keys_out, &perm, st);
+    if (rc != LAPIS_HIP_OK) {
+      (void)hipFree(keys_in);
+      (void)hipFree(val_out);
+      (void)hipFree(idx);
+      return rc;
+    }
+    if (gather_values<T>(perm, val, val_out, nnz, st) != LAPIS_HIP_OK) return fail(hipGetLastError(), "value gather");
+  }
   hipLaunchKernelGGL(colblock_low_word_kernel, dim3((unsigned)ceil_div(nnz, 256)), dim3(256), 0, st, (long long)nnz,
                      keys_out, idx);
   if ((e = hipGetLastError()) != hipSuccess) return fail(e, "index kernel");
   if ((e = hipStreamSynchronize(st)) != hipSuccess) return fail(e, "synchronize");
   (void)hipFree(keys_in);
   (void)hipFree(keys_out);
-  (void)hipFree(temp);
   free_colblock(p);
   p->colblock_group = 0;
+  p->colblock_perm = perm;
+  p->colblock_src_crd = crd;
+  p->colblock_src_val = val;
   {
     const char *stp = getenv("LAPIS_HIP_COLBLOCK_STEPS"), *epl = getenv("LAPIS_HIP_COLBLOCK_EPL"),
                *pad = getenv("LAPIS_HIP_COLBLOCK_PAD");
@@ -447,4 +511,39 @@ extern "C" int lapis_hip_csr_plan_build_colblock(lapis_hip_csr_plan *plan, const
     plan->stats.chunk = 0;
   }
   return rc;
+}
+
+extern "C" int lapis_hip_csr_plan_update_values(lapis_hip_csr_plan *plan, const void *val, int value_bytes,
+                                                lapis_hip_stream_t stream) {
+  LAPIS_CHECK_INIT();
+  LAPIS_REQUIRE(plan, "csr_plan_update_values: null plan");
+  if (!plan->colblock_built) return LAPIS_HIP_OK;  // the CSR kernels read the caller's values on every call
+  LAPIS_REQUIRE(val, "csr_plan_update_values: null values");
+  if (value_bytes != plan->colblock_value_bytes)
+    return set_error(LAPIS_HIP_ERR_PLAN_MISMATCH, "csr_plan_update_values: the copy holds %d-byte values, called with %d",
+                     plan->colblock_value_bytes, value_bytes);
+  hipStream_t st = as_stream(stream);
+  const int rc = value_bytes == 8
+                     ? gather_values<double>(plan->colblock_perm, static_cast<const double *>(val),
+                                             static_cast<double *>(plan->colblock_val), plan->stats.nnz, st)
+                     : gather_values<float>(plan->colblock_perm, static_cast<const float *>(val),
+                                            static_cast<float *>(plan->colblock_val), plan->stats.nnz, st);
+  if (rc == LAPIS_HIP_OK) plan->colblock_src_val = val;
+  return rc;
+}
+
+extern "C" int lapis_hip_csr_plan_analyze(lapis_hip_csr_plan *plan, const int32_t *crd, const void *val, int value_bytes,
+                                          lapis_hip_stream_t stream) {
+  LAPIS_CHECK_INIT();
+  LAPIS_REQUIRE(plan, "csr_plan_analyze: null plan");
+  LAPIS_REQUIRE(value_bytes == 4 || value_bytes == 8, "csr_plan_analyze: value_bytes must be 4 or 8");
+  if (!plan->stats.colblock_recommended || plan->stats.nnz == 0) return LAPIS_HIP_OK;
+  LAPIS_REQUIRE(crd && val, "csr_plan_analyze: null coordinates or values");
+  if (plan->colblock_built && plan->colblock_value_bytes == value_bytes && plan->colblock_src_crd == crd) {
+    plan->stats.kernel = LAPIS_HIP_SPMV_COLBLOCK;  // the copy is there: bring its values up to date
+    return lapis_hip_csr_plan_update_values(plan, val, value_bytes, stream);
+  }
+  const int rc = lapis_hip_csr_plan_build_colblock(plan, crd, val, value_bytes, LAPIS_HIP_COLBLOCK_AUTO, 0, stream);
+  // a matrix the tiling has no room for (too many slices or row blocks) keeps its CSR kernel
+  return rc == LAPIS_HIP_ERR_INVALID_ARGUMENT ? LAPIS_HIP_OK : rc;
 }

@@ -32,6 +32,7 @@
 
 #include <algorithm>
 #include <cstdlib>
+#include <mutex>
 #include <vector>
 
 #include "common.hpp"
@@ -232,12 +233,14 @@ template <typename T, int THREADS, int U, bool NT>
 int launch_colgroup_cfg(const lapis_hip_csr_plan *p, const T *x, T *y, hipStream_t st) {
   auto kernel = spmv_colgroup_kernel<T, THREADS, U, NT>;
   const size_t lds_bytes = sizeof(double) * (size_t)p->colblock_rows + sizeof(int) * ((size_t)p->colblock_nslices + 2);
-  static bool attribute_set = false;  // one per instantiation; more than 64 KB of dynamic LDS has to be asked for
-  if (!attribute_set) {
-    LAPIS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-    attribute_set = true;
-  }
+  // one per instantiation; more than 64 KB of dynamic LDS has to be asked for
+  static std::once_flag attribute_once;
+  static hipError_t attribute_status = hipSuccess;
+  std::call_once(attribute_once, [&] {
+    attribute_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  });
+  LAPIS_HIP_TRY(attribute_status);
   const dim3 grid((unsigned)p->colblock_nunits), block(THREADS);
   hipEvent_t e0, e1;
   if (timing_next_events(&e0, &e1))
@@ -331,15 +334,14 @@ int build_colgroup(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int 
 
   unsigned long long *keys_in = nullptr, *keys_out = nullptr;
   T *val_out = nullptr;
-  unsigned *idx = nullptr;
+  unsigned *idx = nullptr, *perm = nullptr;
   int *tile_ptr = nullptr, *block_range = nullptr, *long_flag = nullptr, *long_rank = nullptr, *long_rows = nullptr,
       *units = nullptr;
-  void *temp = nullptr, *scan_temp = nullptr;
-  size_t temp_bytes = 0, scan_bytes = 0;
+  void *scan_temp = nullptr;
+  size_t scan_bytes = 0;
   auto release = [&](bool all) {
     if (keys_in) (void)hipFree(keys_in);
     if (keys_out) (void)hipFree(keys_out);
-    if (temp) (void)hipFree(temp);
     if (scan_temp) (void)hipFree(scan_temp);
     if (long_flag) (void)hipFree(long_flag);
     if (long_rank) (void)hipFree(long_rank);
@@ -347,6 +349,7 @@ int build_colgroup(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int 
     if (all) {
       if (val_out) (void)hipFree(val_out);
       if (idx) (void)hipFree(idx);
+      if (perm) (void)hipFree(perm);
       if (tile_ptr) (void)hipFree(tile_ptr);
       if (long_rows) (void)hipFree(long_rows);
       if (units) (void)hipFree(units);
@@ -397,7 +400,6 @@ int build_colgroup(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int 
   // 2. sort the entries by (block, column, row in block)
   const size_t ntiles = (size_t)nblocks * ((size_t)nslices + 1);
   if ((e = hipMalloc(&keys_in, sizeof(unsigned long long) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
-  if ((e = hipMalloc(&keys_out, sizeof(unsigned long long) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
   if ((e = hipMalloc(&val_out, sizeof(T) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
   if ((e = hipMalloc(&idx, sizeof(unsigned) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
   if ((e = hipMalloc(&tile_ptr, sizeof(int) * ntiles)) != hipSuccess) return fail(e, "hipMalloc");
@@ -406,13 +408,15 @@ int build_colgroup(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int 
                      col_bits, nblocks_nat, nlong > 0 ? (const int *)long_flag : (const int *)nullptr,
                      (const int *)long_rank, p->pos, crd, keys_in);
   if ((e = hipGetLastError()) != hipSuccess) return fail(e, "key kernel");
-  if ((e = hipcub::DeviceRadixSort::SortPairs(nullptr, temp_bytes, keys_in, keys_out, val, val_out, (int)nnz, 0,
-                                              end_bit, st)) != hipSuccess)
-    return fail(e, "radix sort sizing");
-  if ((e = hipMalloc(&temp, temp_bytes ? temp_bytes : 1)) != hipSuccess) return fail(e, "hipMalloc");
-  if ((e = hipcub::DeviceRadixSort::SortPairs(temp, temp_bytes, keys_in, keys_out, val, val_out, (int)nnz, 0, end_bit,
-                                              st)) != hipSuccess)
-    return fail(e, "radix sort");
+  // the permutation of the sort is kept: lapis_hip_csr_plan_update_values refreshes the copy's values with it
+  {
+    const int rc = sort_keys_with_perm(keys_in, nnz, end_bit, &keys_out, &perm, st);
+    if (rc != LAPIS_HIP_OK) {
+      release(true);
+      return rc;
+    }
+    if (gather_values<T>(perm, val, val_out, nnz, st) != LAPIS_HIP_OK) return fail(hipGetLastError(), "value gather");
+  }
   hipLaunchKernelGGL(colgroup_entry_kernel, dim3((unsigned)ceil_div(nnz, 256)), dim3(256), 0, st, (long long)nnz,
                      row_bits, slice_log2, keys_out, idx);
   if ((e = hipGetLastError()) != hipSuccess) return fail(e, "entry kernel");
@@ -490,6 +494,9 @@ int build_colgroup(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int 
   p->colblock_tile_ptr = tile_ptr;
   p->colblock_idx = idx;
   p->colblock_val = val_out;
+  p->colblock_perm = perm;
+  p->colblock_src_crd = crd;
+  p->colblock_src_val = val;
   p->colblock_value_bytes = (int)sizeof(T);
   p->colblock_col_bits = col_bits;
   p->colblock_slice_log2 = slice_log2;

@@ -25,6 +25,9 @@ struct lapis_hip_csr_plan {
   int colblock_slice_log2;   // columns per x slice = 1 << this
   unsigned *colblock_idx;    // device, uint32[nnz]
   void *colblock_val;        // device, T[nnz]
+  unsigned *colblock_perm;   // device, uint32[nnz]: CSR position of the entry stored at each position of the copy
+  const void *colblock_src_crd;  // the caller's buffers the copy was made from; SpMV calls must pass the same ones
+  const void *colblock_src_val;
   int colblock_steps;        // steps per wavefront trip
   int colblock_epl;          // entries per lane per step (1, 2 or 4)
   int colblock_pad;          // 1: workgroups of 8 wavefronts instead of 4
@@ -67,6 +70,14 @@ template <typename T>
 int launch_colblock(const lapis_hip_csr_plan *plan, const int *pos, const int *crd, const T *val, const T *x, T *y,
                     hipStream_t st);
 void free_colblock(lapis_hip_csr_plan *plan);
+
+// Sorts `nnz` 64-bit keys (bits [0, end_bit)).  On success *keys_out holds the sorted keys and
+// *perm the position each sorted key had before (both device buffers, the caller frees them).
+int sort_keys_with_perm(const unsigned long long *keys_in, int64_t nnz, int end_bit, unsigned long long **keys_out,
+                        unsigned **perm, hipStream_t st);
+// out[i] = val[perm[i]]
+template <typename T>
+int gather_values(const unsigned *perm, const T *val, T *out, int64_t nnz, hipStream_t st);
 
 // y = A x without reading y; defined in spmv.hip.
 int spmv_overwrite_f64(lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, const int32_t *pos,

@@ -550,8 +550,7 @@ int spmv_impl(lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, const int3
                      (long long)s.nrows, (long long)s.ncols, (const void *)plan->pos, (long long)nrows,
                      (long long)ncols, (const void *)pos);
   if (s.nnz == 0) return LAPIS_HIP_OK;
-  LAPIS_REQUIRE(x && (s.kernel == LAPIS_HIP_SPMV_COLBLOCK || (crd && val)),
-                "spmv: null coordinates, values or x with %lld non-zeros", (long long)s.nnz);
+  LAPIS_REQUIRE(x && crd && val, "spmv: null coordinates, values or x with %lld non-zeros", (long long)s.nnz);
   const bool vec = aligned16(crd) && aligned16(val);
   const bool nt = plan->nontemporal;
   switch (s.kernel) {
@@ -572,6 +571,13 @@ int spmv_impl(lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, const int3
       if (!plan->colblock_built || plan->colblock_value_bytes != (int)sizeof(T))
         return set_error(LAPIS_HIP_ERR_PLAN_MISMATCH, "spmv: the plan holds no column-blocked copy for %d-byte values",
                          (int)sizeof(T));
+      // the copy stands in for crd/val: refuse buffers it was not made from (new values in the same
+      // buffer are brought in with lapis_hip_csr_plan_update_values)
+      if (crd != plan->colblock_src_crd || val != plan->colblock_src_val)
+        return set_error(LAPIS_HIP_ERR_PLAN_MISMATCH,
+                         "spmv: the column-blocked copy was made from coordinates %p and values %p, called with %p and %p "
+                         "(lapis_hip_csr_plan_update_values takes new values)",
+                         plan->colblock_src_crd, plan->colblock_src_val, (const void *)crd, (const void *)val);
       return launch_colblock<T>(plan, pos, crd, val, x, y, st);
     default:
       return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT, "spmv: plan holds unknown kernel %d", s.kernel);

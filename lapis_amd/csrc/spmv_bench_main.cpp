@@ -1,8 +1,14 @@
 // SpMV benchmark driver over a MatrixMarket file, the counterpart of the
 // reference's benchmarks/spmv/main.cpp: read the matrix, keep it resident on the
 // device, one warm-up call, then `trials` calls each followed by a fence, print the
-// mean time.  Usage: lapis_spmv_bench matrix.mtx [trials=1000] [kernel]
+// mean time.  Usage: lapis_spmv_bench matrix.mtx [trials=1000] [kernel] [--check] [--dump-y FILE]
 //   kernel: auto (default) | reference | subwarpN | rowblock | nnzsplit | colblock
+//   auto lets the library decide (plan statistics, and with 64 trials or more
+//   lapis_hip_csr_plan_analyze, which builds the column-blocked copy where it pays).
+//   --check       run one product with x = 1, 2, 3, ... and y = 0 before the timing and print
+//                 sum(y) and four entries of y with 17 digits (the reference driver prints
+//                 nothing that can be verified; this is what the tests compare)
+//   --dump-y FILE also write that y as raw doubles
 // Instead of a file, `gen:laplace3d:N` builds the 7-point Laplacian on an N^3 grid
 // (N = 100 is the size of the reference's Laplace3D_100).
 #include <hip/hip_runtime.h>
@@ -162,13 +168,25 @@ void laplace3d(int n, Csr &A) {
 }  // namespace
 
 int main(int argc, const char **argv) {
-  if (argc < 2 || argc > 4) {
-    std::cout << "Expected: matrix file in MatrixMarket format [trials] [kernel]\n";
+  std::vector<std::string> positional;
+  bool check = false;
+  std::string dump_path;
+  for (int i = 1; i < argc; ++i) {
+    const std::string a = argv[i];
+    if (a == "--check") check = true;
+    else if (a == "--dump-y" && i + 1 < argc) dump_path = argv[++i];
+    else if (a.rfind("--", 0) == 0) {
+      std::cerr << "unknown option " << a << "\n";
+      return 1;
+    } else positional.push_back(a);
+  }
+  if (positional.empty() || positional.size() > 3) {
+    std::cout << "Expected: matrix file in MatrixMarket format [trials] [kernel] [--check] [--dump-y FILE]\n";
     return 1;
   }
-  const std::string mfile = argv[1];
-  const int trials = argc > 2 ? std::max(1, atoi(argv[2])) : 1000;
-  const std::string kernel = argc > 3 ? argv[3] : "auto";
+  const std::string mfile = positional[0];
+  const int trials = positional.size() > 1 ? std::max(1, atoi(positional[1].c_str())) : 1000;
+  const std::string kernel = positional.size() > 2 ? positional[2] : "auto";
   CHECK_LAPIS(lapis_hip_init());
   Csr A;
   std::string err;
@@ -215,12 +233,41 @@ int main(int argc, const char **argv) {
     else if (kernel != "auto") {
       std::cerr << "unknown kernel " << kernel << "\n";
       return 1;
+    } else if (trials >= 64) {
+      // enough calls for a column-blocked copy to pay back where the library recommends one
+      CHECK_LAPIS(lapis_hip_csr_plan_analyze(plan, crd, val, 8, nullptr));
     }
     lapis_hip_csr_stats s;
     CHECK_LAPIS(lapis_hip_csr_plan_get_stats(plan, &s));
     std::cout << "rows: min " << s.min_row_len << " mean " << s.mean_row_len << " max " << s.max_row_len
               << "; kernel " << s.kernel << " width " << s.width << "; reference vector length "
               << s.reference_vector_length << "\n";
+  }
+  if (check || !dump_path.empty()) {
+    std::vector<double> hx((size_t)A.ncols), hy((size_t)A.nrows);
+    for (int64_t i = 0; i < A.ncols; ++i) hx[(size_t)i] = (double)(i + 1);
+    CHECK_HIP(hipMemcpy(x, hx.data(), sizeof(double) * hx.size(), hipMemcpyHostToDevice));
+    CHECK_LAPIS(lapis_hip_spmv_csr_f64_i32(plan, A.nrows, A.ncols, pos, crd, val, x, y, nullptr));
+    CHECK_LAPIS(lapis_hip_stream_synchronize(nullptr));
+    CHECK_HIP(hipMemcpy(hy.data(), y, sizeof(double) * hy.size(), hipMemcpyDeviceToHost));
+    double sum = 0.0;
+    for (double v : hy) sum += v;  // ascending index order
+    printf("check: sum(y) = %.17g\n", sum);
+    if (A.nrows > 0) {
+      const int64_t at[4] = {0, A.nrows / 3, A.nrows / 2, A.nrows - 1};
+      for (int64_t i : at) printf("check: y[%lld] = %.17g\n", (long long)i, hy[(size_t)i]);
+    }
+    if (!dump_path.empty()) {
+      FILE *f = fopen(dump_path.c_str(), "wb");
+      if (!f || fwrite(hy.data(), sizeof(double), hy.size(), f) != hy.size()) {
+        std::cerr << "error: cannot write " << dump_path << "\n";
+        return 1;
+      }
+      fclose(f);
+    }
+    // back to the reference driver's state: x and y zero
+    CHECK_HIP(hipMemset(x, 0, sizeof(double) * std::max<int64_t>(A.ncols, 1)));
+    CHECK_HIP(hipMemset(y, 0, sizeof(double) * std::max<int64_t>(A.nrows, 1)));
   }
   // Warmup
   CHECK_LAPIS(lapis_hip_spmv_csr_f64_i32(plan, A.nrows, A.ncols, pos, crd, val, x, y, nullptr));

@@ -53,6 +53,8 @@ _SIGNATURES = {
     "lapis_hip_csr_plan_get_stats": [_vp, ctypes.POINTER(CsrStats)],
     "lapis_hip_csr_plan_destroy": [_vp],
     "lapis_hip_csr_plan_build_colblock": [_vp, _vp, _vp, _int, _int, _int, _vp],
+    "lapis_hip_csr_plan_analyze": [_vp, _vp, _vp, _int, _vp],
+    "lapis_hip_csr_plan_update_values": [_vp, _vp, _int, _vp],
     "lapis_hip_spmv_csr_f64_i32": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp],
     "lapis_hip_spmv_csr_f32_i32": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp],
     "lapis_hip_spmm_csr_f32_i32": [_i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp],
@@ -187,6 +189,17 @@ class CsrPlan:
                                                           COLBLOCK_LAYOUTS[layout], slice_log2_cols,
                                                           _stream(stream)))
         return self.set_kernel(SPMV_COLBLOCK)
+
+    def analyze(self, crd, val, stream=None):
+        """Let the library decide, with the values in hand, whether the column-blocked copy pays; builds it if so."""
+        check(self._lib.lapis_hip_csr_plan_analyze(self._handle, _ptr(crd), _ptr(val), val.element_size(),
+                                                   _stream(stream)))
+        return self
+
+    def update_values(self, val, stream=None):
+        """Refresh the values of the column-blocked copy after ``val`` changed (no-op without a copy)."""
+        check(self._lib.lapis_hip_csr_plan_update_values(self._handle, _ptr(val), val.element_size(), _stream(stream)))
+        return self
 
     def destroy(self):
         if self._handle:

@@ -156,3 +156,40 @@ def test_cg_with_a_column_blocked_plan(gpu, oracle):
     ig, rg = gpu.pcg(plan, n, dpos, dcrd, dval, dev(b), None, 1e-10, 200, x)
     assert rg <= 1e-10 and abs(ig - io) <= 1  # the sums are added in another order: the count may move by one
     assert np.allclose(x.cpu().numpy(), np.ones(n), rtol=1e-8, atol=1e-8)
+
+
+def test_mht_refreshes_a_column_blocked_copy_after_scaling(gpu, oracle, golden):
+    # func @mht scales val in place before its two solves (examples/hitting_times.py:153-179); a plan that
+    # holds a column-blocked copy must multiply with the scaled values, not the ones it was built from
+    pos, crd, val, shape = read_mtx_csr("mht_A.mtx")
+    _, _, dvals, _ = read_mtx_csr("mht_D.mtx")
+    n = shape[0]
+    mask = np.ones(n)
+    mask[3] = 0.0
+    dpos, dcrd, dval = dev(pos), dev(crd), dev(val.copy())
+    plan = gpu.CsrPlan(n, n, dpos, dcrd)
+    plan.build_colblock(dcrd, dval, 2, layout="group")
+    m1 = torch.zeros(n, dtype=torch.float64, device="cuda")
+    m2 = torch.zeros(n, dtype=torch.float64, device="cuda")
+    gpu.mht(plan, n, dpos, dcrd, dval, dev(mask), dev(dvals), 0.99, 1e-10, 20, m1, m2)
+    o1, o2 = oracle.mht(pos, crd, val.copy(), mask, dvals, 0.99, 1e-10, 20)
+    assert np.allclose(m1.cpu().numpy(), o1, rtol=1e-9, atol=1e-12)
+    assert np.allclose(m2.cpu().numpy(), o2, rtol=1e-9, atol=1e-12)
+
+
+def test_cg_without_a_plan_builds_the_copy_when_it_can_pay_back(gpu, oracle):
+    import scipy.sparse as sp
+    R = gen.poisson_random(400000, 2.0, seed=41)
+    B = sp.csr_matrix((np.abs(R.val), R.crd, R.pos), shape=(R.nrows, R.ncols))
+    S = (B + B.T).tocsr()
+    S = (S + sp.diags(np.asarray(S.sum(axis=1)).ravel() + 1.0)).tocsr()
+    S.sort_indices()
+    pos, crd, val = S.indptr.astype(np.int32), S.indices.astype(np.int32), S.data.astype(np.float64)
+    n = S.shape[0]
+    assert S.nnz >= (1 << 20)
+    b = S @ np.ones(n)
+    for maxiter in (100, 20):  # with and without the copy (maxiter < 64 keeps the CSR kernel)
+        x = torch.zeros(n, dtype=torch.float64, device="cuda")
+        ig, rg = gpu.pcg(None, n, dev(pos), dev(crd), dev(val), dev(b), None, 1e-10, maxiter, x)
+        xo, io, ro = oracle.pcg(pos, crd, val, b, np.ones(n), 1e-10, maxiter)
+        assert abs(ig - io) <= 1 and np.allclose(x.cpu().numpy(), xo, rtol=1e-7, atol=1e-9)

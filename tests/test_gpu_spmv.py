@@ -351,3 +351,74 @@ def test_plans_give_back_their_device_memory(gpu):
     torch.cuda.synchronize()
     free1, _ = torch.cuda.mem_get_info()
     assert free0 - free1 < (8 << 20), "plans leak %.1f MB over 15 build/destroy cycles" % ((free0 - free1) / 1e6)
+
+
+@pytest.mark.parametrize("layout", ["group", "wave"])
+def test_column_blocked_copy_follows_value_updates_and_refuses_other_buffers(gpu, oracle, layout):
+    # the reference reads val on every call; a copy has to be told: update_values refreshes it in one
+    # gather pass, and a call with buffers the copy was not made from is refused
+    A = gen.poisson_random(30000, 9.0, seed=21)
+    x = gen.uniform_vector(A.ncols, 22)
+    pos, crd, val, dx = dev(A.pos), dev(A.crd), dev(A.val), dev(x)
+    plan = gpu.CsrPlan(A.nrows, A.ncols, pos, crd)
+    plan.build_colblock(crd, val, 9, layout=layout)
+
+    def run(values):
+        y = torch.zeros(A.nrows, dtype=torch.float64, device="cuda")
+        gpu.spmv(plan, A.nrows, A.ncols, pos, crd, values, dx, y)
+        torch.cuda.synchronize()
+        return y.cpu().numpy()
+
+    def expect(values_host):
+        want = np.zeros(A.nrows)
+        oracle.spmv(A.pos, A.crd, values_host, x, want)
+        return want, oracle.spmv_abs_scale(A.pos, A.crd, values_host, x)
+
+    want, scale = expect(A.val)
+    assert_rows_close(run(val), want, scale, np.float64, "as built")
+    # scale the values in place, as scale_csr of examples/hitting_times.py:51-71 does
+    gpu.scale(-0.375, val)
+    plan.update_values(val)
+    want2, scale2 = expect(A.val * -0.375)
+    assert_rows_close(run(val), want2, scale2, np.float64, "after update_values")
+    # other values in another buffer: refused until update_values is given that buffer
+    other_host = gen.uniform_vector(A.nnz, 23)
+    other = dev(other_host)
+    with pytest.raises(gpu.LapisHipError) as e:
+        run(other)
+    assert e.value.status_name == "LAPIS_HIP_ERR_PLAN_MISMATCH"
+    with pytest.raises(gpu.LapisHipError) as e:
+        y = torch.zeros(A.nrows, dtype=torch.float64, device="cuda")
+        gpu.spmv(plan, A.nrows, A.ncols, pos, dev(A.crd), val, dx, y)  # same coordinates, another buffer
+    assert e.value.status_name == "LAPIS_HIP_ERR_PLAN_MISMATCH"
+    plan.update_values(other)
+    want3, scale3 = expect(other_host)
+    assert_rows_close(run(other), want3, scale3, np.float64, "after update_values with another buffer")
+    plan.destroy()
+
+
+def test_analyze_builds_the_copy_only_where_it_is_recommended(gpu, oracle):
+    # wide uniformly random columns, more than 2^20 non-zeros: the gathers of a chunk range over all of x
+    A = gen.poisson_random(600000, 4.0, seed=31)
+    x = gen.uniform_vector(A.ncols, 32)
+    pos, crd, val = dev(A.pos), dev(A.crd), dev(A.val)
+    plan = gpu.CsrPlan(A.nrows, A.ncols, pos, crd)
+    assert plan.stats()["colblock_recommended"] == 1 and plan.stats()["kernel_name"] in ("rowblock", "nnzsplit")
+    plan.analyze(crd, val)
+    s = plan.stats()
+    assert s["kernel_name"] == "colblock" and s["colblock_layout_name"] == "group"
+    y = torch.zeros(A.nrows, dtype=torch.float64, device="cuda")
+    gpu.spmv(plan, A.nrows, A.ncols, pos, crd, val, dev(x), y)
+    torch.cuda.synchronize()
+    want = np.zeros(A.nrows)
+    oracle.spmv(A.pos, A.crd, A.val, x, want)
+    assert_rows_close(y.cpu().numpy(), want, oracle.spmv_abs_scale(A.pos, A.crd, A.val, x), np.float64, "analyze")
+    plan.analyze(crd, val)  # a second call keeps the copy and refreshes its values
+    assert plan.stats()["kernel_name"] == "colblock"
+    plan.destroy()
+    # a stencil: the gathers stay inside a window L2 holds, the plan keeps its CSR kernel
+    L, _ = gen.config5(scale=(110 / 192) ** 3)
+    lp, lc, lv = dev(L.pos), dev(L.crd), dev(L.val)
+    plan = gpu.CsrPlan(L.nrows, L.ncols, lp, lc)
+    plan.analyze(lc, lv)
+    assert plan.stats()["kernel_name"] == "nnzsplit" and plan.stats()["colblock_layout_name"] is None
