@@ -205,6 +205,29 @@ def run_spmv(args, cfg):
         hms = (time.perf_counter() - t0) / reps * 1e3
         out["host_buffers"] = {"entry": "py_spmv via LAPISModule.spmv (host arrays, H2D + kernel + D2H per call)",
                                "ms_per_call": hms, "GB/s": bytes_step / (hms * 1e-3) / 1e9}
+        if dtype == np.float64:
+            # the opt-in resident path of the same module: matrix bound once, vectors as dual views
+            t0 = time.perf_counter()
+            Ad = mod.bind_csr(A.pos, A.crd, A.val, spec)
+            bind_ms = (time.perf_counter() - t0) * 1e3
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                Ad.spmv(x, yh)
+            mixed_ms = (time.perf_counter() - t0) / reps * 1e3
+            xv, yv = mod.dual_view(x.copy()), mod.dual_view(np.zeros(A.nrows))
+            Ad.spmv(xv, yv)
+            yv.sync_host()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                Ad.spmv(xv, yv)
+            yv.sync_host()
+            rms = (time.perf_counter() - t0) / args.steps * 1e3
+            out["host_buffers"]["resident"] = {
+                "entry": "LAPISModule.bind_csr(...).spmv: matrix, plan and column-blocked copy kept on the device",
+                "bind_ms": bind_ms, "ms_per_call_numpy_vectors": mixed_ms,
+                "ms_per_call_dual_views": rms, "GB/s_dual_views": bytes_step / (rms * 1e-3) / 1e9,
+                "ratio_to_c_abi": rms / ms}
+            Ad.release()
     if published:
         # fenced per-call protocol of the published numbers: one call, one synchronise
         t0 = time.perf_counter()

@@ -75,8 +75,45 @@ typedef struct lapis_csr_specifier {
   int64_t memSizes[3];
 } lapis_csr_specifier;
 
+/* One prebuilt library serves every LAPISModule object of a process, where the
+ * reference has one generated library (and one alives list) per package: the
+ * two calls are counted, and only the last lapis_finalize() frees the results
+ * handed out and finalises the kernel library. */
 void lapis_initialize(void);
 void lapis_finalize(void);
+
+/* ---- operands that stay on the device between calls -----------------------
+ * The role of LAPIS::DualView (LAPISSupport.hpp:136-426), which lets a C++
+ * caller of a generated module keep operands resident across calls
+ * (benchmarks/spmv/main.cpp:42-56), offered through the C ABI: a host buffer
+ * the caller owns paired with a device copy, with the DualView's lazy
+ * modified_host / modified_device flags.  The py_<func> entry points above
+ * keep the reference's copy-per-call behaviour; these are opt-in. */
+typedef struct lapis_dualview_f64 lapis_dualview_f64;
+/* Pairs `n` doubles at `host` (borrowed: they must outlive the view) with a
+ * device allocation; the view starts out modified on the host
+ * (the host-view constructor, LAPISSupport.hpp:214-226). */
+lapis_dualview_f64 *lapis_dualview_f64_create(double *host, int64_t n);
+void lapis_dualview_f64_modify_host(lapis_dualview_f64 *v);   /* modifyHost()  :229 */
+void lapis_dualview_f64_modify_device(lapis_dualview_f64 *v); /* modifyDevice():234 */
+void lapis_dualview_f64_sync_host(lapis_dualview_f64 *v);     /* syncHost()    :251: copies back only if modified on the device */
+void lapis_dualview_f64_sync_device(lapis_dualview_f64 *v);   /* syncDevice()  :271: uploads only if modified on the host */
+void lapis_dualview_f64_destroy(lapis_dualview_f64 *v);
+
+/* A CSR matrix uploaded once: device copies of positions, coordinates and
+ * values, its plan (row statistics -> kernel) and, where the library
+ * recommends it, the column-blocked copy (lapis_hip_csr_plan_analyze). */
+typedef struct lapis_resident_csr lapis_resident_csr;
+lapis_resident_csr *lapis_resident_csr_create(lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd,
+                                              lapis_memref_1d_f64 *val, const lapis_csr_specifier *spec);
+/* new values in the same sparsity pattern (same length and order as at creation) */
+void lapis_resident_csr_update_values(lapis_resident_csr *A, lapis_memref_1d_f64 *val);
+/* func @spmv on resident operands: y += A*x.  x and y are brought to the device
+ * if (and only if) they are marked modified on the host, y is left marked
+ * modified on the device; nothing is copied back and the call does not wait
+ * for the kernel -- lapis_dualview_f64_sync_host(y) does both. */
+void lapis_resident_csr_spmv(lapis_resident_csr *A, lapis_dualview_f64 *x, lapis_dualview_f64 *y);
+void lapis_resident_csr_destroy(lapis_resident_csr *A);
 
 /* func @spmv(A, x, y) -> y of examples/spmv_noalloc.py:9-14 and
  * benchmarks/spmv/spmv.mlir:3-6: y += A*x, y updated in place and returned. */

@@ -7,73 +7,40 @@ example script runs with only its import line changed::
     module_kokkos = backend.compile(moduleText)
     module_kokkos.spmv(rowptrs, colinds, values, ((m, n), (len(rowptrs), len(colinds), len(values))), x, y)
 
-Nothing is compiled at run time: there is no MLIR here.  ``compile`` reads the
-signatures of the module's public functions, checks each one against the catalogue
-of functions the prebuilt gfx950 module implements (the CSR SpMV / SpMM / CG path)
-and binds them.  A module asking for anything else raises, with the reference's own
-message for a failed lowering.
+Nothing is compiled at run time: there is no MLIR here.  ``compile`` reads the module, reduces every
+public function (with the private functions it calls) to a canonical form that keeps the operations and
+their data flow and drops every name (lapis_amd/mlir_text.py), and looks that form up among the
+computations the prebuilt gfx950 module implements (lapis_amd/catalogue.py).  A function binds because
+of WHAT it computes: ``@matvec`` doing ``linalg.matvec`` on a CSR operand binds to the SpMV entry point
+under its own name, while a ``@spmv`` that multiplies by the transpose, or takes a CSC operand, is
+refused with the reference's message for a failed lowering.
 """
 import os
-import re
 
+from . import catalogue as _catalogue
+from . import mlir_text as _mt
 from . import module as _module
 
-# public function name -> (kind, result count); `main` is renamed as the emitter does
-# (TranslateToKokkosCpp.cpp:2351-2355)
-_FUNC_RE = re.compile(r"func\.func\s+(private\s+)?@([A-Za-z_][\w$.]*)\s*\(([^)]*)\)\s*(?:->\s*(\([^)]*\)|[^\s{]+(?:\s*<[^{]*>)?))?", re.S)
+_LOWERING_FAILED = "Lowering to Kokkos dialect failed."
+
+_catalogue_forms = None
+
+
+def _forms():
+    """canonical form -> entry point of the prebuilt module"""
+    global _catalogue_forms
+    if _catalogue_forms is None:
+        forms = {}
+        for entry, text in _catalogue.entries():
+            forms[_mt.Canonicalizer(text).canonical("f")] = entry
+        _catalogue_forms = forms
+    return _catalogue_forms
 
 
 def _public_functions(text):
-    funcs = []
-    for m in _FUNC_RE.finditer(text):
-        if m.group(1):
-            continue
-        name = m.group(2)
-        args = [a.strip() for a in _split_top(m.group(3))] if m.group(3).strip() else []
-        funcs.append((name, args, bool(m.group(4))))
-    return funcs
-
-
-def _split_top(s):
-    out, depth, cur = [], 0, ""
-    for ch in s:
-        if ch in "<([{":
-            depth += 1
-        elif ch in ">)]}":
-            depth -= 1
-        if ch == "," and depth == 0:
-            out.append(cur)
-            cur = ""
-        else:
-            cur += ch
-    if cur.strip():
-        out.append(cur)
-    return out
-
-
-def _classify(arg):
-    """'csr' for a 2-D tensor with an encoding attribute, 'vec'/'mat' for dense tensors, 'scalar' otherwise."""
-    m = re.search(r"tensor<([^>]*)", arg)
-    if not m:
-        return "scalar"
-    body = m.group(1)
-    dims = body.count("x")
-    if "#" in arg.split("tensor<", 1)[1]:
-        return "csr" if dims == 2 else ("csrv" if dims == 3 else "sparse")
-    return {1: "vec", 2: "mat"}.get(dims, "dense%d" % dims)
-
-
-# what the prebuilt module implements: name -> argument kinds
-_CATALOGUE = {
-    "spmv": ["csr", "vec", "vec"],
-    "lapis_main": ["csr", "vec"],
-    "pcg": ["csr", "vec", "vec", "scalar", "scalar"],
-    "spmm": ["csr", "mat", "mat"],
-    "plus_norm": ["vec", "vec"],
-    "mht": ["csr", "vec", "vec", "scalar", "scalar", "scalar"],
-    "normalize_mom2": ["vec", "vec"],
-    "pte_local_bspmm": ["csrv", "dense3"],
-}
+    """(name, argument kinds, has a result) of the module's public functions."""
+    c = _mt.Canonicalizer(text)
+    return [(f.name, c.signature(f)[0], bool(f.results)) for f in c.public()]
 
 
 class KokkosBackend:
@@ -90,37 +57,57 @@ class KokkosBackend:
         self.package_name = "lapis_package" if index_instance == 0 else "lapis_package_" + str(index_instance)
 
     def bind(self, moduleText):
-        """Names of the module's public functions after checking them against the catalogue."""
-        funcs = _public_functions(moduleText)
-        if not funcs:
-            raise Exception("Lowering to Kokkos dialect failed.")
-        names = []
+        """{method name: entry point of the prebuilt module} for the module's public functions.
+
+        The method name is the function's own (``main`` becomes ``lapis_main`` as in the emitter,
+        TranslateToKokkosCpp.cpp:2351-2355); the entry point is found by what the function computes."""
+        try:
+            c = _mt.Canonicalizer(moduleText)
+            public = c.public()
+        except _mt.ParseError as e:
+            raise Exception(_LOWERING_FAILED + "\nthe module text could not be read: %s" % e)
+        if not public:
+            raise Exception(_LOWERING_FAILED)
+        bound = {}
         self.unbound = []
-        for name, args, has_result in funcs:
-            bound = "lapis_main" if name == "main" else name
-            kinds = [_classify(a) for a in args]
-            if bound not in _CATALOGUE and not has_result:
-                # a helper that returns nothing (the sparse_tensor.print wrapper of examples/bspmm.py:54-58):
-                # compiled by the reference, not implemented here; the rest of the module still binds
-                self.unbound.append(bound)
-                continue
-            if bound not in _CATALOGUE or _CATALOGUE[bound] != kinds:
-                raise Exception("Lowering to Kokkos dialect failed.\nfunction @%s(%s) is outside the CSR SpMV / SpMM / CG "
-                                "path the gfx950 module implements" % (name, ", ".join(kinds)))
-            if ("csr" in kinds or "csrv" in kinds) and not self.decompose_tensors:
-                raise Exception("Lowering to Kokkos dialect failed.\n@%s takes a sparse tensor: pass decompose_tensors=True "
-                                "(positions, coordinates, values and the storage specifier as separate arguments)" % name)
-            names.append(bound)
-        return names
+        for f in public:
+            method = "lapis_main" if f.name == "main" else f.name
+            kinds, results = c.signature(f)
+            if f.body is None:
+                raise Exception(_LOWERING_FAILED + "\n@%s is declared without a body" % f.name)
+            try:
+                form = c.canonical(f.name)
+            except _mt.ParseError as e:
+                raise Exception(_LOWERING_FAILED + "\n@%s could not be read: %s" % (f.name, e))
+            entry = _forms().get(form)
+            if entry is None:
+                if not results:
+                    # a helper that returns nothing (the sparse_tensor.print wrapper of examples/bspmm.py:54-58):
+                    # compiled by the reference, not implemented here; the rest of the module still binds
+                    self.unbound.append(method)
+                    continue
+                sparse = [k for k in kinds if k.startswith("sparse(")]
+                why = ("its sparse operand is stored as %s; the module implements CSR and CSRV with 32-bit positions "
+                       "and coordinates" % sparse[0][7:-1]) if sparse else \
+                    "what it computes is not one of the CSR SpMV / SpMM / CG functions the gfx950 module implements"
+                raise Exception("%s\nfunction @%s(%s): %s" % (_LOWERING_FAILED, f.name, ", ".join(kinds), why))
+            if any(k.startswith(("csr:", "csrv:")) for k in kinds) and not self.decompose_tensors:
+                raise Exception(_LOWERING_FAILED + "\n@%s takes a sparse tensor: pass decompose_tensors=True "
+                                "(positions, coordinates, values and the storage specifier as separate arguments)" % f.name)
+            bound[method] = entry
+        return bound
 
     def compile(self, module):
         moduleText = str(module)
         if self.dump_mlir:
             print("== High-Level ==")
             print(moduleText)
-        names = self.bind(moduleText)
+        bound = self.bind(moduleText)
         mod = _module.LAPISModule()
-        mod.bound_functions = names
+        mod.bound_functions = sorted(bound)
+        for method, entry in bound.items():
+            if method != entry:
+                setattr(mod, method, getattr(mod, entry))  # the function's own name, the entry its body calls for
         for name in self.unbound:
             def _not_implemented(*args, _name=name, **kwargs):
                 raise NotImplementedError("@%s is outside the CSR SpMV / SpMM / CG path the gfx950 module implements" % _name)

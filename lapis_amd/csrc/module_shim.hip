@@ -6,6 +6,8 @@
 // keep-alive list for results handed to Python (LAPISSupport.hpp:101-120).
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -205,19 +207,118 @@ void spmm_entry(MM **ret0, lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd, M
 
 extern "C" void lapis_initialize(void) {
   std::lock_guard<std::mutex> lock(g_mutex);
-  if (g_initialized) return;  // `if (!Kokkos::is_initialized())`: repeated calls do nothing
+  // `if (!Kokkos::is_initialized())`: only the first call initialises; every call is counted, because
+  // this one library stands in for all the generated packages of a process
+  if (g_initialized++ > 0) return;
   check(lapis_hip_init(), "lapis_hip_init");
-  g_initialized = 1;
 }
 
 extern "C" void lapis_finalize(void) {
   std::lock_guard<std::mutex> lock(g_mutex);
+  if (g_initialized == 0) return;
+  if (--g_initialized > 0) return;  // another module object is alive: its results must stay valid
   for (void *p : g_alives) free(p);  // LAPIS::alives.clear()
   g_alives.clear();
-  if (g_initialized) {
-    lapis_hip_finalize();
-    g_initialized = 0;
-  }
+  lapis_hip_finalize();
+}
+
+// ---- resident operands ----------------------------------------------------------------------------
+
+struct lapis_dualview_f64 {
+  double *host = nullptr;
+  double *dev = nullptr;
+  int64_t n = 0;
+  bool modified_host = false;
+  bool modified_device = false;
+};
+
+struct lapis_resident_csr {
+  int64_t nrows = 0, ncols = 0, nnz = 0;
+  int32_t *pos = nullptr, *crd = nullptr;
+  double *val = nullptr;
+  lapis_hip_csr_plan *plan = nullptr;
+};
+
+extern "C" lapis_dualview_f64 *lapis_dualview_f64_create(double *host, int64_t n) {
+  if (n < 0 || (n > 0 && !host)) module_abort("dualview: null host buffer or negative length");
+  lapis_dualview_f64 *v = new lapis_dualview_f64();
+  v->host = host;
+  v->n = n;
+  if (n > 0) check_hip(hipMalloc(&v->dev, sizeof(double) * (size_t)n), "hipMalloc");
+  v->modified_host = true;
+  return v;
+}
+
+extern "C" void lapis_dualview_f64_modify_host(lapis_dualview_f64 *v) { v->modified_host = true; }
+extern "C" void lapis_dualview_f64_modify_device(lapis_dualview_f64 *v) { v->modified_device = true; }
+
+extern "C" void lapis_dualview_f64_sync_host(lapis_dualview_f64 *v) {
+  if (!v->modified_device) return;
+  // hipMemcpy on the null stream waits for the kernels queued there before it copies
+  if (v->n > 0) check_hip(hipMemcpy(v->host, v->dev, sizeof(double) * (size_t)v->n, hipMemcpyDeviceToHost), "device-to-host copy");
+  v->modified_device = false;
+}
+
+extern "C" void lapis_dualview_f64_sync_device(lapis_dualview_f64 *v) {
+  if (!v->modified_host) return;
+  if (v->n > 0) check_hip(hipMemcpy(v->dev, v->host, sizeof(double) * (size_t)v->n, hipMemcpyHostToDevice), "host-to-device copy");
+  v->modified_host = false;
+}
+
+extern "C" void lapis_dualview_f64_destroy(lapis_dualview_f64 *v) {
+  if (!v) return;
+  if (v->dev) (void)hipFree(v->dev);
+  delete v;
+}
+
+extern "C" lapis_resident_csr *lapis_resident_csr_create(lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd,
+                                                         lapis_memref_1d_f64 *val, const lapis_csr_specifier *spec) {
+  int32_t *hpos = host_data(pos, 1, "positions");
+  int32_t *hcrd = host_data(crd, 1, "coordinates");
+  double *hval = host_data(val, 1, "values");
+  const CsrArgs a = csr_args(pos, crd, val->sizes[0], spec);
+  lapis_resident_csr *A = new lapis_resident_csr();
+  A->nrows = a.nrows;
+  A->ncols = a.ncols;
+  A->nnz = a.nnz;
+  check_hip(hipMalloc(&A->pos, sizeof(int32_t) * ((size_t)a.nrows + 1)), "hipMalloc");
+  check_hip(hipMalloc(&A->crd, sizeof(int32_t) * (size_t)std::max<int64_t>(a.nnz, 1)), "hipMalloc");
+  check_hip(hipMalloc(&A->val, sizeof(double) * (size_t)std::max<int64_t>(a.nnz, 1)), "hipMalloc");
+  check_hip(hipMemcpy(A->pos, hpos, sizeof(int32_t) * ((size_t)a.nrows + 1), hipMemcpyHostToDevice), "host-to-device copy");
+  check_hip(hipMemcpy(A->crd, hcrd, sizeof(int32_t) * (size_t)a.nnz, hipMemcpyHostToDevice), "host-to-device copy");
+  check_hip(hipMemcpy(A->val, hval, sizeof(double) * (size_t)a.nnz, hipMemcpyHostToDevice), "host-to-device copy");
+  check(lapis_hip_csr_plan_create(&A->plan, a.nrows, a.ncols, a.nnz, A->pos, A->crd, 8, nullptr),
+        "lapis_hip_csr_plan_create");
+  // a resident matrix is there to be multiplied many times: let the library build the copy it recommends
+  check(lapis_hip_csr_plan_analyze(A->plan, A->crd, A->val, 8, nullptr), "lapis_hip_csr_plan_analyze");
+  return A;
+}
+
+extern "C" void lapis_resident_csr_update_values(lapis_resident_csr *A, lapis_memref_1d_f64 *val) {
+  double *hval = host_data(val, 1, "values");
+  if (val->sizes[0] < A->nnz) module_abort("update_values: fewer values than the matrix has non-zeros");
+  check_hip(hipMemcpy(A->val, hval, sizeof(double) * (size_t)A->nnz, hipMemcpyHostToDevice), "host-to-device copy");
+  check(lapis_hip_csr_plan_update_values(A->plan, A->val, 8, nullptr), "lapis_hip_csr_plan_update_values");
+}
+
+extern "C" void lapis_resident_csr_spmv(lapis_resident_csr *A, lapis_dualview_f64 *x, lapis_dualview_f64 *y) {
+  if (x->n < A->ncols) module_abort("x is shorter than the number of columns");
+  if (y->n < A->nrows) module_abort("y is shorter than the number of rows");
+  if (x == y) module_abort("x and y must be different views");
+  lapis_dualview_f64_sync_device(x);
+  lapis_dualview_f64_sync_device(y);
+  check(lapis_hip_spmv_csr_f64_i32(A->plan, A->nrows, A->ncols, A->pos, A->crd, A->val, x->dev, y->dev, nullptr),
+        "lapis_hip_spmv_csr_f64_i32");
+  y->modified_device = true;
+}
+
+extern "C" void lapis_resident_csr_destroy(lapis_resident_csr *A) {
+  if (!A) return;
+  lapis_hip_csr_plan_destroy(A->plan);
+  if (A->pos) (void)hipFree(A->pos);
+  if (A->crd) (void)hipFree(A->crd);
+  if (A->val) (void)hipFree(A->val);
+  delete A;
 }
 
 extern "C" void py_spmv(lapis_memref_1d_f64 **ret0, lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd,

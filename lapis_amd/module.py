@@ -31,6 +31,93 @@ def _flatten_specifier(spec):
     return flat
 
 
+class DualView:
+    """A numpy array paired with a device copy that stays allocated between calls: the role of
+    LAPIS::DualView (LAPISSupport.hpp:136-426) with its lazy modified-host / modified-device flags.
+    ``host`` is the numpy side; after writing to it call ``modify_host()``; ``sync_host()`` brings a
+    result back (and waits for the kernels that produce it)."""
+
+    def __init__(self, lib, array):
+        self._lib = lib
+        self.host = numpy.require(array, dtype=numpy.float64, requirements=['C', 'W'])
+        self._handle = ctypes.c_void_p(lib.lapis_dualview_f64_create(self.host.ctypes.data_as(ctypes.c_void_p),
+                                                                     ctypes.c_int64(self.host.shape[0])))
+
+    def modify_host(self):
+        self._lib.lapis_dualview_f64_modify_host(self._handle)
+        return self
+
+    def sync_host(self):
+        self._lib.lapis_dualview_f64_sync_host(self._handle)
+        return self.host
+
+    def sync_device(self):
+        self._lib.lapis_dualview_f64_sync_device(self._handle)
+        return self
+
+    def release(self):
+        if self._handle:
+            self._lib.lapis_dualview_f64_destroy(self._handle)
+            self._handle = None
+
+    def __del__(self):
+        try:
+            self.release()
+        except Exception:
+            pass
+
+
+class ResidentCsr:
+    """A CSR matrix uploaded once (``LAPISModule.bind_csr``): device copies, plan and, where the library
+    recommends it, the column-blocked copy are reused by every ``spmv``."""
+
+    def __init__(self, module, pos, crd, val, spec):
+        self._module = module  # keeps the library initialised for as long as the matrix lives
+        self._lib = module.libHandle
+        pos = numpy.require(pos, dtype=numpy.int32, requirements=['C'])
+        crd = numpy.require(crd, dtype=numpy.int32, requirements=['C'])
+        val = numpy.require(val, dtype=numpy.float64, requirements=['C'])
+        flat = _flatten_specifier(spec)
+        self.shape = (int(flat[0]), int(flat[1]))
+        self._handle = ctypes.c_void_p(self._lib.lapis_resident_csr_create(
+            ctypes.pointer(rt.get_ranked_memref_descriptor(pos)), ctypes.pointer(rt.get_ranked_memref_descriptor(crd)),
+            ctypes.pointer(rt.get_ranked_memref_descriptor(val)), flat.ctypes.data_as(ctypes.c_void_p)))
+
+    def update_values(self, val):
+        val = numpy.require(val, dtype=numpy.float64, requirements=['C'])
+        self._lib.lapis_resident_csr_update_values(self._handle, ctypes.pointer(rt.get_ranked_memref_descriptor(val)))
+
+    def spmv(self, x, y):
+        """y += A x.  With ``DualView`` operands nothing crosses PCIe and the call returns before the kernel
+        has run (``y.sync_host()`` fetches the result); numpy operands are copied in and out as
+        ``LAPISModule.spmv`` does, and the updated ``y`` is returned."""
+        if isinstance(x, DualView) and isinstance(y, DualView):
+            self._lib.lapis_resident_csr_spmv(self._handle, x._handle, y._handle)
+            return y
+        xv = x if isinstance(x, DualView) else DualView(self._lib, x)
+        yv = y if isinstance(y, DualView) else DualView(self._lib, y)
+        self._lib.lapis_resident_csr_spmv(self._handle, xv._handle, yv._handle)
+        out = yv.sync_host()
+        if out is not y and isinstance(y, numpy.ndarray):
+            y[...] = out  # numpy.require had to copy (dtype or layout): keep the in-place contract
+            out = y
+        for v, given in ((xv, x), (yv, y)):
+            if v is not given:
+                v.release()
+        return out
+
+    def release(self):
+        if self._handle:
+            self._lib.lapis_resident_csr_destroy(self._handle)
+            self._handle = None
+
+    def __del__(self):
+        try:
+            self.release()
+        except Exception:
+            pass
+
+
 class LAPISModule:
     def __init__(self, libPath=None):
         libPath = libPath or DEFAULT_MODULE_PATH
@@ -40,12 +127,34 @@ class LAPISModule:
         self.libHandle = ctypes.CDLL(libPath)
         self.libHandle.lapis_initialize.restype = None
         self.libHandle.lapis_finalize.restype = None
+        self.libHandle.lapis_dualview_f64_create.restype = ctypes.c_void_p
+        self.libHandle.lapis_dualview_f64_create.argtypes = [ctypes.c_void_p, ctypes.c_int64]
+        for fn in ("modify_host", "modify_device", "sync_host", "sync_device", "destroy"):
+            f = getattr(self.libHandle, "lapis_dualview_f64_" + fn)
+            f.restype, f.argtypes = None, [ctypes.c_void_p]
+        self.libHandle.lapis_resident_csr_create.restype = ctypes.c_void_p
+        self.libHandle.lapis_resident_csr_update_values.restype = None
+        self.libHandle.lapis_resident_csr_update_values.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+        self.libHandle.lapis_resident_csr_spmv.restype = None
+        self.libHandle.lapis_resident_csr_spmv.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+        self.libHandle.lapis_resident_csr_destroy.restype = None
+        self.libHandle.lapis_resident_csr_destroy.argtypes = [ctypes.c_void_p]
         self.libHandle.lapis_initialize()
 
     def __del__(self):
         handle = getattr(self, "libHandle", None)
         if handle is not None:
             handle.lapis_finalize()
+
+    # ---- operands that stay on the device (opt-in; the methods below copy per call as the reference does) ----
+    def bind_csr(self, param0, param1, param2, param3):
+        """Upload a CSR matrix (positions, coordinates, values, storage specifier) once; the returned
+        object's ``spmv(x, y)`` reuses the device copies, the plan and the column-blocked layout."""
+        return ResidentCsr(self, param0, param1, param2, param3)
+
+    def dual_view(self, array):
+        """A float64 vector that keeps a device copy between calls (see ``DualView``)."""
+        return DualView(self.libHandle, array)
 
     # func @spmv(A, x, y) -> y          (examples/spmv_noalloc.py:9, benchmarks/spmv/spmv.mlir)
     def spmv(self, param0, param1, param2, param3, param4, param5):

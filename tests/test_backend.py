@@ -1,66 +1,93 @@
-"""The KokkosBackend-shaped front door: signature parsing and catalogue checks (CPU only)."""
+"""The KokkosBackend-shaped front door: functions are bound by what they compute (CPU only)."""
+import os
+import re
+
 import pytest
 
+import modules_mlir as M
+from lapis_amd import mlir_text
 from lapis_amd.KokkosBackend import KokkosBackend, _public_functions
 
-SPMV_NOALLOC = """
-#sparse = #sparse_tensor.encoding<{ map = (d0, d1) -> (d0 : dense, d1 : compressed), posWidth = 32, crdWidth = 32 }>
-module {
-  func.func @spmv(%A: tensor<?x?xf64, #sparse>, %x: tensor<?xf64>, %y: tensor<?xf64>) -> tensor<?xf64> {
-    %0 = linalg.matvec ins(%A, %x: tensor<?x?xf64, #sparse>, tensor<?xf64>) outs(%y : tensor<?xf64>) -> tensor<?xf64>
-    return %0 : tensor<?xf64>
-  }
-}"""
-
-PCG = """
-module {
-  func.func private @spmv(%A: tensor<?x?xf64, #sparse>, %x: tensor<?xf64>, %ydst: tensor<?xf64>) -> tensor<?xf64> { }
-  func.func private @dot(%x: tensor<?xf64>, %y: tensor<?xf64>) -> f64 { }
-  func.func @pcg(%A: tensor<?x?xf64, #sparse>, %b: tensor<?xf64>, %dinv: tensor<?xf64>, %tol: f64, %maxiter: index) -> (tensor<?xf64>, index, f64) { }
-}"""
+REFERENCE_EXAMPLES = "/root/reference/examples"
 
 
-def test_public_functions_skip_private_helpers():
-    assert [f[0] for f in _public_functions(PCG)] == ["pcg"]
-    assert [f[0] for f in _public_functions(SPMV_NOALLOC)] == ["spmv"]
+def test_public_functions_and_their_argument_kinds():
+    assert _public_functions(M.PCG) == [("pcg", ["csr:f64", "vec:f64", "vec:f64", "f64", "index"], True)]
+    assert _public_functions(M.SPMV) == [("spmv", ["csr:f64", "vec:f64", "vec:f64"], True)]
+    # `tensor<?xindex>` is a vector whatever letters its element type holds; an inline encoding with `->` parses
+    text = "func.func @f(%a: tensor<?xindex>, %b: tensor<4x?xf32>, %c: index) -> index { return %c : index }"
+    assert _public_functions(text)[0][1] == ["vec:index", "mat:f32", "index"]
+    assert _public_functions(M.MATVEC_OTHER_NAME)[0][1] == ["csr:f64", "vec:f64", "vec:f64"]
 
 
-def test_bind_accepts_the_path_and_renames_main():
+def test_bind_goes_by_the_body_not_by_the_name():
     b = KokkosBackend(decompose_tensors=True)
-    assert b.bind(SPMV_NOALLOC) == ["spmv"]
-    assert b.bind(PCG) == ["pcg"]
-    torch_mv = "func.func @main(%arg0: tensor<5x5xf64, #sparse>, %arg1: tensor<5xf64>) -> tensor<5xf64> { }"
-    assert b.bind(torch_mv) == ["lapis_main"]
+    assert b.bind(M.SPMV) == {"spmv": "spmv"}
+    assert b.bind(M.MATVEC_OTHER_NAME) == {"apply_operator": "spmv"}
+    assert b.bind(M.PCG) == {"pcg": "pcg"}
+    assert b.bind(M.PCG.replace("@pcg(", "@solve(")) == {"solve": "pcg"}
+    torch_mv = """
+    #sparse = #sparse_tensor.encoding<{ map = (d0, d1) -> (d0 : dense, d1 : compressed), posWidth = 32, crdWidth = 32 }>
+    func.func @main(%arg0: tensor<5x5xf64, #sparse>, %arg1: tensor<5xf64>) -> tensor<5xf64> {
+      %cst = arith.constant 0.000000e+00 : f64
+      %0 = tensor.empty() : tensor<5xf64>
+      %1 = linalg.fill ins(%cst : f64) outs(%0 : tensor<5xf64>) -> tensor<5xf64>
+      %2 = linalg.matvec ins(%arg0, %arg1 : tensor<5x5xf64, #sparse>, tensor<5xf64>) outs(%1 : tensor<5xf64>) -> tensor<5xf64>
+      return %2 : tensor<5xf64>
+    }"""
+    assert b.bind(torch_mv) == {"lapis_main": "lapis_main"}  # `main` is renamed as the emitter does
 
 
-BSPMM = """
-#csrv = #sparse_tensor.encoding<{ map = (d0, d1, d2) -> (d0 : dense, d1 : compressed, d2 : dense), posWidth = 32, crdWidth = 32}>
-module {
-  func.func @pte_local_bspmm(%A: tensor<?x?x?xf32, #csrv>,
-    %B: tensor<?x?x?xf32>) ->  tensor<?x?x?xf32>
-  { }
-  func.func @print_csrv(%A: tensor<?x?x?xf32, #csrv>)
-  { }
-}"""
+def test_a_known_name_with_a_foreign_body_is_refused():
+    b = KokkosBackend(decompose_tensors=True)
+    for text, why in ((M.SPMV_TRANSPOSED, "what it computes"), (M.SPMV_CSC, "d1 : dense, d0 : compressed"),
+                      (M.SPMV_WIDE_INDEX, "width other than 32"), (M.PCG_WRONG_SIGN, "what it computes")):
+        with pytest.raises(Exception, match="Lowering to Kokkos dialect failed") as e:
+            b.bind(text)
+        assert why in str(e.value)
+    with pytest.raises(Exception, match="Lowering to Kokkos dialect failed"):
+        b.bind("func.func @gemm(%a: tensor<?x?xf64>, %b: tensor<?x?xf64>, %c: tensor<?x?xf64>) -> tensor<?x?xf64> {\n"
+               "  %0 = linalg.matmul ins(%a, %b : tensor<?x?xf64>, tensor<?x?xf64>) outs(%c : tensor<?x?xf64>) -> tensor<?x?xf64>\n"
+               "  return %0 : tensor<?x?xf64>\n}")  # dense x dense
+    with pytest.raises(Exception, match="declared without a body"):
+        b.bind("func.func @spmv(%x: tensor<?xf64>) -> tensor<?xf64>")
+    with pytest.raises(Exception, match="decompose_tensors"):
+        KokkosBackend().bind(M.SPMV)
+    with pytest.raises(Exception):
+        b.bind("module { }")
 
 
 def test_bind_takes_the_batched_csrv_product_and_sets_its_print_helper_aside():
     # shape of the module in examples/bspmm.py:10-60
     b = KokkosBackend(decompose_tensors=True)
-    assert b.bind(BSPMM) == ["pte_local_bspmm"]
+    assert b.bind(M.BSPMM) == {"pte_local_bspmm": "pte_local_bspmm"}
     assert b.unbound == ["print_csrv"]
 
 
-def test_bind_rejects_what_the_module_does_not_implement():
-    b = KokkosBackend(decompose_tensors=True)
-    with pytest.raises(Exception, match="Lowering to Kokkos dialect failed"):
-        b.bind("func.func @gemm(%a: tensor<?x?xf64>, %b: tensor<?x?xf64>) -> tensor<?x?xf64> { }")
-    with pytest.raises(Exception, match="Lowering to Kokkos dialect failed"):
-        b.bind("func.func @spmv(%x: tensor<?xf64>) -> tensor<?xf64> { }")  # right name, wrong signature
-    with pytest.raises(Exception, match="decompose_tensors"):
-        KokkosBackend().bind(SPMV_NOALLOC)
-    with pytest.raises(Exception):
-        b.bind("module { }")
+def test_canonical_form_ignores_names_comments_and_constant_order():
+    a = mlir_text.Canonicalizer(M.SPMV).canonical("spmv")
+    b = mlir_text.Canonicalizer(M.MATVEC_OTHER_NAME).canonical("apply_operator")
+    assert a == b
+    moved = M.PCG.replace("    %f0 = arith.constant 0.0 : f64\n    %f1 = arith.constant 1.0 : f64\n",
+                          "    %f1 = arith.constant 1.0 : f64\n    %unused = arith.constant -1.0 : f64\n    %f0 = arith.constant 0.0 : f64\n")
+    assert moved != M.PCG
+    assert mlir_text.Canonicalizer(moved).canonical("pcg") == mlir_text.Canonicalizer(M.PCG).canonical("pcg")
+    # swapping the operands of a division is another computation
+    other = M.PCG.replace("arith.divf %rzn, %rzold", "arith.divf %rzold, %rzn")
+    assert mlir_text.Canonicalizer(other).canonical("pcg") != mlir_text.Canonicalizer(M.PCG).canonical("pcg")
+
+
+@pytest.mark.skipif(not os.path.isdir(REFERENCE_EXAMPLES), reason="the reference tree is not on this machine")
+@pytest.mark.parametrize("example, expected", [
+    ("spmv_noalloc.py", {"spmv": "spmv"}), ("pcg_solve.py", {"pcg": "pcg"}),
+    ("multiple_results.py", {"plus_norm": "plus_norm"}),
+    ("hitting_times.py", {"mht": "mht", "normalize_mom2": "normalize_mom2"}),
+    ("bspmm.py", {"pte_local_bspmm": "pte_local_bspmm"})])
+def test_module_texts_of_the_reference_examples_bind(example, expected):
+    # the example files are read as text; nothing of them is imported or run
+    src = open(os.path.join(REFERENCE_EXAMPLES, example)).read()
+    text = re.search(r'moduleText\s*=\s*"""(.*?)"""', src, re.S).group(1)
+    assert KokkosBackend(decompose_tensors=True).bind(text) == expected
 
 
 def test_constructor_mirrors_the_reference():

@@ -161,3 +161,127 @@ def test_non_contiguous_memref_aborts_like_kokkos_abort():
     proc = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
     assert proc.returncode != 0 and "survived" not in proc.stdout
     assert "not contiguous" in proc.stderr
+
+
+# ---- through KokkosBackend.compile(moduleText), as the example scripts do ----------------------------
+
+def test_compile_binds_spmv_by_its_body_and_reproduces_the_literal_answer(gpu, golden):
+    import modules_mlir as M
+    from lapis_amd import KokkosBackend
+    g = golden["spmv_noalloc"]
+    rowptrs, colinds = np.array(g["pos"], np.int32), np.array(g["crd"], np.int32)
+    values = np.array(g["val"], np.double)
+    backend = KokkosBackend.KokkosBackend(decompose_tensors=True)
+    module_kokkos = backend.compile(M.SPMV)
+    y = np.zeros(5)
+    module_kokkos.spmv(rowptrs, colinds, values, ((5, 5), (len(rowptrs), len(colinds), len(values))), np.ones(5), y)
+    assert np.allclose(y, [1.1, 2.2, -19, -1, 0])  # examples/spmv_noalloc.py:31
+    # the same computation under another name binds to the same kernel, under ITS name
+    other = backend.compile(M.MATVEC_OTHER_NAME)
+    y2 = np.zeros(5)
+    other.apply_operator(rowptrs, colinds, values, ((5, 5), (6, 8, 8)), np.ones(5), y2)
+    assert np.array_equal(y2, y)
+    # the right name on the wrong computation never reaches a kernel
+    with pytest.raises(Exception, match="Lowering to Kokkos dialect failed"):
+        backend.compile(M.SPMV_TRANSPOSED)
+
+
+def test_compile_binds_pcg_and_matches_scipy_on_nos4(gpu):
+    import modules_mlir as M
+    from lapis_amd import KokkosBackend
+    pos, crd, val, shape = read_mtx_csr("nos4.mtx")
+    A = sp.csr_matrix((val, crd, pos), shape=shape)
+    n = A.shape[0]
+    b = A @ np.ones(n)
+    dinv = 1.0 / A.diagonal()
+    module_kokkos = KokkosBackend.KokkosBackend(decompose_tensors=True).compile(M.PCG)
+    (x, numiter, relres) = module_kokkos.pcg(A.indptr, A.indices, A.data, ((n, n), (n + 1, A.nnz, A.nnz)), b, dinv,
+                                              1e-10, 40)
+    [x_scipy, info] = scipy_cg(A, b, np.zeros((n)), rtol=1e-10, maxiter=40, M=sp.diags(dinv))
+    assert np.allclose(x, x_scipy)  # the acceptance check of examples/pcg_solve.py:134
+
+
+def test_two_modules_share_the_library_and_outlive_each_other(gpu, golden):
+    # every compile() returns a new module object over the one prebuilt library: dropping one of them must
+    # neither free the results of the other nor shut the library down under it
+    import gc
+    import modules_mlir as M
+    from lapis_amd import KokkosBackend
+    g = golden["spmv_noalloc"]
+    rowptrs, colinds = np.array(g["pos"], np.int32), np.array(g["crd"], np.int32)
+    values = np.array(g["val"], np.double)
+    backend = KokkosBackend.KokkosBackend(decompose_tensors=True)
+    torch_mv = M.SPMV.replace("@spmv(%A: tensor<?x?xf64, #sparse>, %x: tensor<?xf64>, %y: tensor<?xf64>)",
+                              "@main(%A: tensor<?x?xf64, #sparse>, %x: tensor<?xf64>)")
+    first = backend.compile(M.SPMV)
+    second = backend.compile(M.SPMV)
+    kept = second.lapis_main(rowptrs, colinds, values, ((5, 5), (6, 8, 8)), np.ones(5))  # module-owned result
+    want = kept.copy()
+    del first
+    gc.collect()
+    junk = [np.full(5, 7.0) for _ in range(64)]  # reuse freed heap blocks, if any were freed
+    assert np.array_equal(kept, want) and np.allclose(want, g["y_expected"])
+    y = np.zeros(5)
+    second.spmv(rowptrs, colinds, values, ((5, 5), (6, 8, 8)), np.ones(5), y)  # the library is still initialised
+    assert np.allclose(y, g["y_expected"])
+    del junk
+
+
+# ---- operands that stay on the device -----------------------------------------------------------------
+
+def test_resident_matrix_and_dual_views(gpu, oracle):
+    from lapis_amd.module import LAPISModule
+    mod = LAPISModule()
+    A = gen.poisson_random(50000, 7.0, seed=61)
+    x = gen.uniform_vector(A.ncols, 62)
+    spec = ((A.nrows, A.ncols), (A.nrows + 1, A.nnz, A.nnz))
+    Ad = mod.bind_csr(A.pos, A.crd, A.val, spec)
+    want = np.zeros(A.nrows)
+    oracle.spmv(A.pos, A.crd, A.val, x, want)
+    scale = oracle.spmv_abs_scale(A.pos, A.crd, A.val, x)
+    # numpy operands: copied per call, y updated in place like LAPISModule.spmv
+    y = np.zeros(A.nrows)
+    ret = Ad.spmv(x, y)
+    assert ret is y and np.all(np.abs(y - want) <= 1e-12 * np.maximum(scale, 1e-300))
+    # dual views: nothing is copied until asked for; two products accumulate on the device
+    xv, yv = mod.dual_view(x.copy()), mod.dual_view(np.zeros(A.nrows))
+    Ad.spmv(xv, yv)
+    Ad.spmv(xv, yv)
+    assert np.all(yv.host == 0.0)  # the host half is stale until sync_host
+    got = yv.sync_host()
+    assert np.all(np.abs(got - 2 * want) <= 2e-12 * np.maximum(scale, 1e-300))
+    # a host-side change is seen only after modify_host, as with the DualView it stands for
+    xv.host[:] = 2 * x
+    yv.host[:] = 0.0
+    yv.modify_host()
+    Ad.spmv(xv, yv)
+    assert np.all(np.abs(yv.sync_host() - want) <= 1e-12 * np.maximum(scale, 1e-300))  # still the old x
+    xv.modify_host()
+    yv.host[:] = 0.0
+    yv.modify_host()
+    Ad.spmv(xv, yv)
+    assert np.all(np.abs(yv.sync_host() - 2 * want) <= 2e-12 * np.maximum(scale, 1e-300))
+    # new values in the same pattern
+    Ad.update_values(-A.val)
+    y3 = np.zeros(A.nrows)
+    Ad.spmv(x, y3)
+    assert np.all(np.abs(y3 + want) <= 1e-12 * np.maximum(scale, 1e-300))
+    Ad.release()
+
+
+def test_resident_matrix_gets_the_column_blocked_copy_where_recommended(gpu, oracle):
+    from lapis_amd.module import LAPISModule
+    mod = LAPISModule()
+    A = gen.poisson_random(600000, 4.0, seed=63)
+    x = gen.uniform_vector(A.ncols, 64)
+    Ad = mod.bind_csr(A.pos, A.crd, A.val, ((A.nrows, A.ncols), (A.nrows + 1, A.nnz, A.nnz)))
+    y = np.zeros(A.nrows)
+    Ad.spmv(x, y)
+    want = np.zeros(A.nrows)
+    oracle.spmv(A.pos, A.crd, A.val, x, want)
+    scale = oracle.spmv_abs_scale(A.pos, A.crd, A.val, x)
+    assert np.all(np.abs(y - want) <= 1e-12 * np.maximum(scale, 1e-300))
+    Ad.update_values(0.5 * A.val)  # refreshes the copy through the kept permutation
+    y2 = np.zeros(A.nrows)
+    Ad.spmv(x, y2)
+    assert np.all(np.abs(y2 - 0.5 * want) <= 1e-12 * np.maximum(scale, 1e-300))
