@@ -48,6 +48,65 @@ def traffic_from_profiles(kernel_key, kernel_ms):
     return entry["hbm_bytes_per_launch"]
 
 
+def calibrate_gather(full=False):
+    """Rates of the two things a column-blocked SpMV launch spends its time on, measured with the library's
+    calibration kernel (lapis_hip_calibrate_gather): streaming the matrix, and gathering x from L2 one
+    128-byte line per request.  On this chip the two do not overlap: the times ADD.  With `full` the whole
+    table (merge factors 1..16, the three cache levels) is returned as well."""
+    import torch
+    from lapis_amd import hip
+    gathers = 1 << 26
+    stream = torch.zeros(1 << 27, dtype=torch.float64, device="cuda")  # 1 GiB: 12 bytes per gather fit
+    x = torch.zeros(1 << 23, dtype=torch.float64, device="cuda")       # 64 MB window at most
+    sink = torch.zeros(4096, dtype=torch.float64, device="cuda")
+    l2 = 1 << 20
+    only_stream = hip.calibrate_gather(None, 0, 0, stream, gathers, sink)
+    only_gather = hip.calibrate_gather(x, l2, 1, None, gathers, sink)
+    both = hip.calibrate_gather(x, l2, 1, stream, gathers, sink)
+    stream_rate = only_stream["stream_bytes"] / (only_stream["ms"] * 1e-3)  # bytes/s
+    line_rate = only_gather["gathers"] / (only_gather["ms"] * 1e-3)          # 128-byte lines/s
+    out = {"stream_only_ms": only_stream["ms"], "stream_TB_per_s": stream_rate / 1e12,
+           "gather_only_ms": only_gather["ms"], "gather_lines_G_per_s": line_rate / 1e9,
+           "both_ms": both["ms"], "sum_of_parts_ms": only_stream["ms"] + only_gather["ms"],
+           "window": "1 MB of x (L2 resident)", "gathers": only_gather["gathers"],
+           "stream_bytes": only_stream["stream_bytes"]}
+    if full:
+        table = []
+        for window, label in ((16 << 10, "16 KB (vector cache)"), (l2, "1 MB (L2)"), (64 << 20, "64 MB (HBM)")):
+            for lanes in (1, 2, 4, 8, 16):
+                for with_stream in (False, True):
+                    if window != l2 and lanes != 1:
+                        continue
+                    r = hip.calibrate_gather(x, window, lanes, stream if with_stream else None, gathers, sink)
+                    lines = r["gathers"] / lanes
+                    table.append({"window": label, "lanes_per_line": lanes, "stream": with_stream, "ms": r["ms"],
+                                  "gather_lines_G_per_s": lines / (r["ms"] * 1e-3) / 1e9,
+                                  "predicted_ms": (r["stream_bytes"] / stream_rate + lines / line_rate) * 1e3
+                                  if window == l2 else None})
+        out["table"] = table
+    del stream, x, sink
+    return out
+
+
+def colgroup_request_floor(stats, A, cal, value_bytes):
+    """Floor of the workgroup column-blocked kernel from the calibrated rates: the matrix copy streamed once
+    plus one L2 request per distinct 128-byte line of x a tile touches.  A block of R rows puts
+    d = R * mean_row_len * (128 / value_bytes) / ncols entries into every line of x on average; with columns
+    drawn uniformly a wave instruction's 64 column-sorted neighbours merge into (1 - exp(-d)) / d requests per
+    entry.  Returned only for matrices without long rows (those go to blocks of their own)."""
+    import math
+    if stats["max_row_len"] >= max(2048.0, 16.0 * stats["mean_row_len"]):
+        return None
+    rows = 16384 if A.nrows > 8192 else (8192 if A.nrows > 4096 else 4096)
+    d = rows * stats["mean_row_len"] * (128.0 / value_bytes) / max(1, A.ncols)
+    per_entry = (1.0 - math.exp(-d)) / d if d > 1e-9 else 1.0
+    lines = A.nnz * per_entry
+    copy_bytes = A.nnz * (4 + value_bytes)
+    floor_ms = (copy_bytes / (cal["stream_TB_per_s"] * 1e12) + lines / (cal["gather_lines_G_per_s"] * 1e9)) * 1e3
+    return {"entries_per_line": d, "requests_per_entry": per_entry, "gather_lines_per_launch": lines,
+            "streamed_bytes_per_launch": copy_bytes, "floor_ms": floor_ms}
+
+
 def cpu_baseline_spmv(A, x, budget_s=12.0):
     """The OpenMP restatement of the reference loop nest, timed on this host's cores."""
     from oracle.oracle import Oracle
@@ -167,6 +226,17 @@ def run_spmv(args, cfg):
                      "traffic": traffic_from_profiles("%s_config%d" % (family, cfg), kt["mean_ms"]) if cfg else None,
                      "kernel_ms_mean": kt["mean_ms"], "kernel_ms_min": kt["min_ms"], "launches_timed": kt["count"]},
     }
+    if family == "colgroup" and not args.no_calibration:
+        cal = calibrate_gather(full=args.calibrate_gather)
+        floor = colgroup_request_floor(stats, A, cal, np.dtype(dtype).itemsize)
+        out["calibration"] = cal
+        if floor:
+            # what bounds this kernel is not HBM: its traffic is 1.35 x algorithmic at 3.7 TB/s.  It is the
+            # requests its compute units can keep in flight; see calibrate_gather().
+            out["roofline"]["secondary"] = dict(floor, bound="line_requests_in_flight", achieved_ms=kt["mean_ms"],
+                                                frac=floor["floor_ms"] / kt["mean_ms"],
+                                                model="stream_bytes / stream rate + gather lines / line rate "
+                                                      "(calibrated in this run; the two do not overlap)")
     if args.graph or cfg == 1:
         # Launch-bound sizes: the same calls captured once into a HIP graph (10 per graph) and
         # replayed, which takes the Python and launch overhead of each call out of the loop.
@@ -371,6 +441,10 @@ def main():
                     help="also time the calls replayed from a HIP graph (always done for config 1)")
     ap.add_argument("--host-buffers", action="store_true",
                     help="also time the generated-module entry point, which takes host arrays (PCIe-inclusive)")
+    ap.add_argument("--calibrate-gather", action="store_true",
+                    help="print the whole gather/stream calibration table (merge factors, cache levels) instead of "
+                         "the three rows the secondary roofline needs")
+    ap.add_argument("--no-calibration", action="store_true", help="skip the gather/stream calibration launches")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch the library's copy kernel on 1 GiB three times, the known-size reference "
                          "that rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")

@@ -64,6 +64,20 @@ int lapis_hip_stream_synchronize(lapis_hip_stream_t stream);
 int lapis_hip_kernel_timing_start(int capacity);
 int lapis_hip_kernel_timing_stop(int *count, double *mean_ms, double *min_ms, double *max_ms);
 
+/* Measurement only (`bench.py --calibrate-gather`): one launch in the shape of the
+ * column-blocked SpMV kernels -- one workgroup of 512 threads per compute unit,
+ * each thread per step streaming three 16-byte vectors from `stream_buf` (12 bytes
+ * per gather, what crd + val of an fp64 non-zero take; NULL = no stream) and
+ * gathering four doubles from the first `window_bytes` of `x`, with
+ * `lanes_per_line` neighbouring lanes of a wave instruction in one 128-byte line
+ * (0 = no gathers).  Returns the best of five timed launches in `elapsed_ms` and
+ * what one launch did.  `sink` takes one double per compute unit.  The reference
+ * has no counterpart; its table of measured SpMV times is
+ * benchmarks/plots/spmv.csv.  Synchronises `stream`. */
+int lapis_hip_calibrate_gather(const double *x, int64_t window_bytes, int lanes_per_line, const void *stream_buf,
+                               int64_t stream_bytes, int64_t gathers, double *sink, double *elapsed_ms,
+                               double *gathers_done, double *stream_bytes_done, lapis_hip_stream_t stream);
+
 /* ---- CSR plan: the team/vector loop-mapping decision ---------------------- */
 
 /* Which kernel a plan launches for SpMV. */

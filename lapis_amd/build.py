@@ -21,7 +21,8 @@ LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(CSRC, "build")
 INCLUDE = os.path.join(ROOT, "include")
 
-KERNEL_SOURCES = ["runtime.hip", "spmv.hip", "colblock.hip", "colgroup.hip", "spmm.hip", "blas1.hip", "cg.hip"]
+KERNEL_SOURCES = ["runtime.hip", "spmv.hip", "colblock.hip", "colgroup.hip", "spmm.hip", "blas1.hip", "cg.hip",
+                  "calibrate.hip"]
 SHIM_SOURCES = ["module_shim.hip"]
 
 KERNEL_LIB = os.path.join(LIBDIR, "liblapis_hip.so")

@@ -48,6 +48,8 @@ _SIGNATURES = {
     "lapis_hip_kernel_timing_start": [_int],
     "lapis_hip_kernel_timing_stop": [ctypes.POINTER(_int), ctypes.POINTER(_dbl), ctypes.POINTER(_dbl),
                                      ctypes.POINTER(_dbl)],
+    "lapis_hip_calibrate_gather": [_vp, _i64, _int, _vp, _i64, _i64, _vp, ctypes.POINTER(_dbl), ctypes.POINTER(_dbl),
+                                   ctypes.POINTER(_dbl), _vp],
     "lapis_hip_csr_plan_create": [ctypes.POINTER(_vp), _i64, _i64, _i64, _vp, _vp, _int, _vp],
     "lapis_hip_csr_plan_set_kernel": [_vp, _int, _int],
     "lapis_hip_csr_plan_get_stats": [_vp, ctypes.POINTER(CsrStats)],
@@ -247,6 +249,18 @@ def dot(x, y, result, init_value=0.0, stream=None):
     fn = getattr(lib, "lapis_hip_dot_%s" % _suffix(x))
     check(fn(int(x.shape[0]), _ptr(x), _ptr(y), init_value, _ptr(result), _stream(stream)))
     return result
+
+
+def calibrate_gather(x, window_bytes, lanes_per_line, stream_buf, gathers, sink, stream=None):
+    """One row of the gather/stream calibration table: dict(ms, gathers, stream_bytes)."""
+    lib = init()
+    ms, done, sbytes = _dbl(0.0), _dbl(0.0), _dbl(0.0)
+    check(lib.lapis_hip_calibrate_gather(_ptr(x) if x is not None else None, window_bytes, lanes_per_line,
+                                         _ptr(stream_buf) if stream_buf is not None else None,
+                                         stream_buf.numel() * stream_buf.element_size() if stream_buf is not None else 0,
+                                         gathers, _ptr(sink), ctypes.byref(ms), ctypes.byref(done), ctypes.byref(sbytes),
+                                         _stream(stream)))
+    return {"ms": ms.value, "gathers": done.value, "stream_bytes": sbytes.value}
 
 
 def dot_noalloc(x, y, result, init_value=0.0, stream=None):
