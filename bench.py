@@ -318,18 +318,34 @@ def run_spmm(args):
     import torch
     from lapis_amd import generators as gen
     from lapis_amd import hip
-    A, B = gen.config4()
-    k = B.shape[1]
+    k = args.k
+    if args.workload:
+        # structure of one of the reference's published SpMV matrices (fp64 in the table), here as the
+        # sparse operand of an fp32 SpMM: a matrix WITH column locality, beside config 4 which has none
+        A = gen.PUBLISHED[args.workload][0]()
+        A = gen.CSR(A.nrows, A.ncols, A.pos, A.crd, A.val.astype(np.float32))
+        B = gen.uniform_matrix(A.ncols, k, 4005).astype(np.float32)
+        name = "%s (structure of the reference's published matrix) as fp32 SpMM operand, B %dx%d row-major" % (
+            args.workload, A.ncols, k)
+    else:
+        A, B = gen.config4()
+        if k != B.shape[1]:
+            B = gen.uniform_matrix(A.ncols, k, 4005).astype(np.float32)
+        name = "config4: SpMM fp32, A 1048576^2 with 32 nnz/row, B 1048576x%d row-major" % k
     dev = lambda a: torch.from_numpy(a).cuda()
     pos, crd, val, dB = dev(A.pos), dev(A.crd), dev(A.val), dev(B)
     C = torch.zeros(A.nrows, k, dtype=torch.float32, device="cuda")
+    if args.spmm_kernel != "auto":
+        os.environ["LAPIS_HIP_SPMM_KERNEL"] = args.spmm_kernel
+    plan = hip.CsrPlan(A.nrows, A.ncols, pos, crd, value_bytes=4)  # its band statistics pick the kernel
+    stats = plan.stats()
     for _ in range(args.warmup):
-        hip.spmm(A.nrows, A.ncols, pos, crd, val, dB, C)
+        hip.spmm(A.nrows, A.ncols, pos, crd, val, dB, C, plan=plan)
     torch.cuda.synchronize()
     hip.kernel_timing_start(args.steps)
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        hip.spmm(A.nrows, A.ncols, pos, crd, val, dB, C)
+        hip.spmm(A.nrows, A.ncols, pos, crd, val, dB, C, plan=plan)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     kt = hip.kernel_timing_stop()
@@ -341,14 +357,17 @@ def run_spmm(args):
         "metric": "CSR x dense SpMM fp32 achieved HBM GB/s", "value": bytes_step / (ms * 1e-3) / 1e9, "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "config4: SpMM fp32, A 1048576^2 with 32 nnz/row, B 1048576x64 row-major",
-                   "nrows": A.nrows, "nnz": A.nnz, "k": k, "seed": 4004, "algorithmic_bytes_per_step": bytes_step},
+        "config": {"workload": name, "nrows": A.nrows, "nnz": A.nnz, "k": k, "seed": 4004,
+                   "algorithmic_bytes_per_step": bytes_step, "spmm_kernel": args.spmm_kernel,
+                   "near_diagonal_fraction": stats["near_diagonal_fraction"], "mean_row_len": stats["mean_row_len"]},
         "pct_of_hbm_peak": 100.0 * bytes_step / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "gflops": 2.0 * A.nnz * k / (ms * 1e-3) / 1e9,
-        "roofline": {"bound": "hbm", "kernel": "spmm_wave_row_kernel<float,16>", "achieved": achieved,
+        "roofline": {"bound": "hbm", "kernel": "spmm kernel chosen by the plan (wave-per-row or LDS-staged row block)",
+                     "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": traffic_from_profiles("spmm_config4", kt["mean_ms"]), "kernel_ms_mean": kt["mean_ms"],
-                     "launches_timed": kt["count"]},
+                     "traffic": traffic_from_profiles("spmm_config4", kt["mean_ms"])
+                     if not args.workload and k == 64 else None, "kernel_ms_mean": kt["mean_ms"],
+                     "kernel_ms_min": kt["min_ms"], "launches_timed": kt["count"]},
     }
     if not args.no_cpu:
         from oracle.oracle import Oracle
@@ -436,6 +455,9 @@ def main():
     ap.add_argument("--colblock-layout", choices=["auto", "wave", "group"], default="auto",
                     help="layout of the column-blocked copy (auto = group)")
     ap.add_argument("--width", type=int, default=0, help="lanes per row with --kernel subwarp (0 = the reference's rule)")
+    ap.add_argument("--k", type=int, default=64, help="columns of B for the SpMM workloads (config 4)")
+    ap.add_argument("--spmm-kernel", choices=["auto", "wave", "group", "lds"], default="auto",
+                    help="SpMM kernel: the plan's choice, the wavefront-per-row kernel, or the LDS-staged row-block kernel")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--graph", action="store_true",
                     help="also time the calls replayed from a HIP graph (always done for config 1)")
@@ -451,7 +473,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
-    if args.workload:
+    if args.workload and args.config != 4:
         args.config = 1  # takes the SpMV path; run_spmv swaps the matrix in
     if args.steps is None:
         args.steps = {1: 1000, 2: 200, 3: 200, 4: 20, 5: 100}[args.config]

@@ -120,6 +120,10 @@ typedef struct lapis_hip_csr_stats {
   int32_t colblock_recommended;
   /* enum lapis_hip_colblock_layout of the copy this plan holds, 0 if none */
   int32_t colblock_layout;
+  /* fraction of the non-zeros with |column - row| <= 32, 64, 128, 256: how much of the
+   * matrix sits in a band around the diagonal (what the LDS-staged SpMM kernel can
+   * serve from its staged window of B); -1 if crd was not given */
+  double near_diagonal_fraction[4];
 } lapis_hip_csr_stats;
 
 typedef struct lapis_hip_csr_plan lapis_hip_csr_plan;
@@ -231,6 +235,26 @@ int lapis_hip_spmm_csr_f32_i32(int64_t nrows, int64_t ncols, int64_t k, const in
 int lapis_hip_spmm_csr_f64_i32(int64_t nrows, int64_t ncols, int64_t k, const int32_t *pos,
                                const int32_t *crd, const double *val, const double *B, int64_t ldb,
                                double *C, int64_t ldc, lapis_hip_stream_t stream);
+
+/* The same product with the plan's statistics deciding the kernel.
+ *   group per row: matrices with short, even rows (mean <= 256, longest <= 4 x mean)
+ *     whose columns stay local (the B rows a stretch of 1024 non-zeros touches fit the
+ *     L2s: stencils, meshes).  64/LPR rows per wavefront at a time, one group of lanes
+ *     per row, no cross-lane reduction: 1.1x-3.9x faster than the kernel below there.
+ *   wavefront per row: everything else, and `plan == NULL` (the entry points above).
+ *   LDS-staged row block: a workgroup stages the rows of B of its block's diagonal
+ *     window in LDS with coalesced 128-bit loads and serves the non-zeros inside the
+ *     window from LDS.  Built and kept selectable (LAPIS_HIP_SPMM_KERNEL=lds) but never
+ *     chosen: on MI355X it measured 1.6x-2.4x slower than group per row on the
+ *     stencil and FEM matrices it is meant for.
+ * The reference chooses between its loop mappings by strategy name
+ * (Pipelines/Passes.h:41-56), never by looking at the columns. */
+int lapis_hip_spmm_csr_f32_i32_plan(const lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, int64_t k,
+                                    const int32_t *pos, const int32_t *crd, const float *val, const float *B,
+                                    int64_t ldb, float *C, int64_t ldc, lapis_hip_stream_t stream);
+int lapis_hip_spmm_csr_f64_i32_plan(const lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, int64_t k,
+                                    const int32_t *pos, const int32_t *crd, const double *val, const double *B,
+                                    int64_t ldb, double *C, int64_t ldc, lapis_hip_stream_t stream);
 
 /* Batched CSRV product of examples/bspmm.py:22-50 (out(n1,dh,nh) += A(n1,n2,nh) * V(n2,dh,nh)):
  * A is CSR over (n1, n2), each non-zero carries nh values (val has nnz*nh entries). */

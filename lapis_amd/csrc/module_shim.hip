@@ -178,20 +178,20 @@ void spmm_entry(MM **ret0, lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd, M
   {
     DeviceMirror<int32_t> dpos(hpos, (size_t)a.nrows + 1), dcrd(hcrd, (size_t)a.nnz);
     DeviceMirror<T> dval(hval, (size_t)a.nnz), dB(hB, (size_t)(a.ncols * k)), dC(hC, (size_t)(a.nrows * k));
-    // the plan is built only for its structure check: a bad coordinate must not reach the kernel
+    // the plan checks the structure (a bad coordinate must not reach the kernel) and its statistics pick the kernel
     lapis_hip_csr_plan *plan = nullptr;
     check(lapis_hip_csr_plan_create(&plan, a.nrows, a.ncols, a.nnz, dpos.dev, dcrd.dev, (int)sizeof(T), nullptr),
           "lapis_hip_csr_plan_create");
-    lapis_hip_csr_plan_destroy(plan);
     int rc;
     if (sizeof(T) == 8)
-      rc = lapis_hip_spmm_csr_f64_i32(a.nrows, a.ncols, k, dpos.dev, dcrd.dev, (const double *)dval.dev,
-                                      (const double *)dB.dev, k, (double *)dC.dev, k, nullptr);
+      rc = lapis_hip_spmm_csr_f64_i32_plan(plan, a.nrows, a.ncols, k, dpos.dev, dcrd.dev, (const double *)dval.dev,
+                                           (const double *)dB.dev, k, (double *)dC.dev, k, nullptr);
     else
-      rc = lapis_hip_spmm_csr_f32_i32(a.nrows, a.ncols, k, dpos.dev, dcrd.dev, (const float *)dval.dev,
-                                      (const float *)dB.dev, k, (float *)dC.dev, k, nullptr);
+      rc = lapis_hip_spmm_csr_f32_i32_plan(plan, a.nrows, a.ncols, k, dpos.dev, dcrd.dev, (const float *)dval.dev,
+                                           (const float *)dB.dev, k, (float *)dC.dev, k, nullptr);
     check(rc, "lapis_hip_spmm_csr");
     check(lapis_hip_stream_synchronize(nullptr), "stream synchronize");
+    lapis_hip_csr_plan_destroy(plan);
     dC.sync_host();
   }
   (*ret0)->basePtr = hC;

@@ -301,6 +301,7 @@ struct DeviceStats {
   unsigned long long empty_rows;
   double sum_sq;
   unsigned long long span_sum;  // sum over 1024-non-zero chunks of (max column - min column)
+  unsigned long long near[4];   // non-zeros with |column - row| <= 32, 64, 128, 256
 };
 
 __global__ __launch_bounds__(256) void row_stats_kernel(int nrows, const int *__restrict__ pos,
@@ -360,6 +361,37 @@ __global__ __launch_bounds__(256) void crd_range_kernel(long long nnz, int ncols
     if (bad) atomicOr(&st->bad, 2);
     atomicAdd(&st->span_sum, (unsigned long long)((long long)mx - (long long)mn));
   }
+}
+
+// How much of the matrix lies in a band around the diagonal: one thread per row
+// (a plan-time pass; the reads are not coalesced), block totals added with one atomic each.
+__global__ __launch_bounds__(256) void band_stats_kernel(int nrows, long long nnz, const int *__restrict__ pos,
+                                                         const int *__restrict__ crd, DeviceStats *st) {
+  __shared__ unsigned long long tot[4];
+  if (threadIdx.x < 4) tot[threadIdx.x] = 0ull;
+  __syncthreads();
+  const long long r = (long long)blockIdx.x * 256 + threadIdx.x;
+  unsigned cnt[4] = {0u, 0u, 0u, 0u};
+  if (r < nrows) {
+    // the structure has not been validated yet: stay inside crd whatever pos holds
+    const long long first = std::max<long long>(0, pos[r]), last = std::min<long long>(nnz, pos[r + 1]);
+    for (long long j = first; j < last; ++j) {
+      const long long d = (long long)crd[j] - r;
+      const long long a = d < 0 ? -d : d;
+      cnt[0] += a <= 32;
+      cnt[1] += a <= 64;
+      cnt[2] += a <= 128;
+      cnt[3] += a <= 256;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    unsigned v = cnt[i];
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    if ((threadIdx.x & 63) == 0 && v) atomicAdd(&tot[i], (unsigned long long)v);
+  }
+  __syncthreads();
+  if (threadIdx.x < 4 && tot[threadIdx.x]) atomicAdd(&st->near[threadIdx.x], tot[threadIdx.x]);
 }
 
 template <int CH>
@@ -639,7 +671,7 @@ extern "C" int lapis_hip_csr_plan_create(lapis_hip_csr_plan **out, int64_t nrows
     return set_error(LAPIS_HIP_ERR_BAD_CSR, "csr_plan_create: pos[0]=%d pos[n]=%d, expected 0 and nnz=%lld",
                      ends[0], ends[1], (long long)nnz);
 
-  DeviceStats init{INT32_MAX, 0, 0, 0, 0ull, 0.0, 0ull};
+  DeviceStats init{INT32_MAX, 0, 0, 0, 0ull, 0.0, 0ull, {0ull, 0ull, 0ull, 0ull}};
   DeviceStats host = init;
   if (nrows > 0) {
     DeviceStats *dstats = nullptr;
@@ -654,6 +686,11 @@ extern "C" int lapis_hip_csr_plan_create(lapis_hip_csr_plan **out, int64_t nrows
       const int blocks = (int)ceil_div(ceil_div(nnz, 1024), 4);
       hipLaunchKernelGGL(crd_range_kernel, dim3(blocks), dim3(256), 0, st, (long long)nnz, (int)ncols, crd,
                          dstats);
+      e = hipGetLastError();
+    }
+    if (e == hipSuccess && crd && nnz > 0) {
+      hipLaunchKernelGGL(band_stats_kernel, dim3((unsigned)ceil_div(nrows, 256)), dim3(256), 0, st, (int)nrows,
+                         (long long)nnz, pos, crd, dstats);
       e = hipGetLastError();
     }
     if (e == hipSuccess) e = hipMemcpyAsync(&host, dstats, sizeof(host), hipMemcpyDeviceToHost, st);
@@ -680,6 +717,7 @@ extern "C" int lapis_hip_csr_plan_create(lapis_hip_csr_plan **out, int64_t nrows
   s.mean_row_len = nrows ? (double)nnz / (double)nrows : 0.0;
   s.var_row_len = nrows ? std::max(0.0, host.sum_sq / (double)nrows - s.mean_row_len * s.mean_row_len) : 0.0;
   s.mean_chunk_col_span = (crd && nnz > 0) ? (double)host.span_sum / (double)ceil_div(nnz, 1024) : -1.0;
+  for (int i = 0; i < 4; ++i) s.near_diagonal_fraction[i] = (crd && nnz > 0) ? (double)host.near[i] / (double)nnz : -1.0;
   // The column-blocked copy pays when the gathers of a chunk wander over more of x
   // than an XCD's L2 keeps (4 MB, shared with the streamed arrays) and the matrix is
   // large enough for the extra launch work not to matter.

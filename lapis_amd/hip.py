@@ -32,10 +32,12 @@ class CsrStats(ctypes.Structure):
                 ("mean_row_len", _dbl), ("var_row_len", _dbl), ("mean_chunk_col_span", _dbl),
                 ("reference_hint", _i64), ("reference_vector_length", ctypes.c_int32),
                 ("kernel", ctypes.c_int32), ("width", ctypes.c_int32), ("chunk", ctypes.c_int32),
-                ("colblock_recommended", ctypes.c_int32), ("colblock_layout", ctypes.c_int32)]
+                ("colblock_recommended", ctypes.c_int32), ("colblock_layout", ctypes.c_int32),
+                ("near_diagonal_fraction", _dbl * 4)]
 
     def as_dict(self):
         d = {k: getattr(self, k) for k, _ in self._fields_}
+        d["near_diagonal_fraction"] = list(self.near_diagonal_fraction)
         d["kernel_name"] = KERNEL_NAMES.get(self.kernel, "?")
         d["colblock_layout_name"] = {0: None, 1: "wave", 2: "group"}.get(self.colblock_layout)
         return d
@@ -61,6 +63,8 @@ _SIGNATURES = {
     "lapis_hip_spmv_csr_f32_i32": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp],
     "lapis_hip_spmm_csr_f32_i32": [_i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp],
     "lapis_hip_spmm_csr_f64_i32": [_i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp],
+    "lapis_hip_spmm_csr_f32_i32_plan": [_vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp],
+    "lapis_hip_spmm_csr_f64_i32_plan": [_vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp],
     "lapis_hip_bspmm_csrv_f32_i32": [_i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp],
     "lapis_hip_dot_f64": [_i64, _vp, _vp, _dbl, _vp, _vp],
     "lapis_hip_dot_f32": [_i64, _vp, _vp, _flt, _vp, _vp],
@@ -233,11 +237,16 @@ def spmv(plan, nrows, ncols, pos, crd, val, x, y, stream=None):
     return y
 
 
-def spmm(nrows, ncols, pos, crd, val, B, C, stream=None):
-    """C += A B with row-major B (ncols x k) and C (nrows x k)."""
+def spmm(nrows, ncols, pos, crd, val, B, C, stream=None, plan=None):
+    """C += A B with row-major B (ncols x k) and C (nrows x k); with a plan its statistics pick the kernel."""
     lib = init()
-    fn = getattr(lib, "lapis_hip_spmm_csr_%s_i32" % _suffix(val))
     k = int(C.shape[1])
+    if plan is not None:
+        fn = getattr(lib, "lapis_hip_spmm_csr_%s_i32_plan" % _suffix(val))
+        check(fn(plan.handle, nrows, ncols, k, _ptr(pos), _ptr(crd), _ptr(val), _ptr(B), int(B.stride(0)), _ptr(C),
+                 int(C.stride(0)), _stream(stream)))
+        return C
+    fn = getattr(lib, "lapis_hip_spmm_csr_%s_i32" % _suffix(val))
     check(fn(nrows, ncols, k, _ptr(pos), _ptr(crd), _ptr(val), _ptr(B), int(B.stride(0)), _ptr(C), int(C.stride(0)),
              _stream(stream)))
     return C

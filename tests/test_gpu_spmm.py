@@ -10,14 +10,16 @@ from lapis_amd import generators as gen
 pytestmark = pytest.mark.gpu
 
 
-def _check(gpu, oracle, A, B, C_in, dtype, what):
+def _check(gpu, oracle, A, B, C_in, dtype, what, plan=False):
     print("case", what, flush=True)
     want = C_in.copy()
     oracle.spmm(A.pos, A.crd, A.val, B, want)
     absA = sp.csr_matrix((np.abs(A.val).astype(np.float64), A.crd, A.pos), shape=(A.nrows, A.ncols))
     scale = absA @ np.abs(B).astype(np.float64) + np.abs(C_in)
     C = dev(C_in)
-    gpu.spmm(A.nrows, A.ncols, dev(A.pos), dev(A.crd), dev(A.val), dev(B), C)
+    dpos, dcrd = dev(A.pos), dev(A.crd)
+    the_plan = gpu.CsrPlan(A.nrows, A.ncols, dpos, dcrd, value_bytes=np.dtype(dtype).itemsize) if plan else None
+    gpu.spmm(A.nrows, A.ncols, dpos, dcrd, dev(A.val), dev(B), C, plan=the_plan)
     torch.cuda.synchronize()
     got = C.cpu().numpy().astype(np.float64)
     err = np.abs(got - want.astype(np.float64))
@@ -26,7 +28,7 @@ def _check(gpu, oracle, A, B, C_in, dtype, what):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
-@pytest.mark.parametrize("k", [64, 1, 2, 3, 8, 32, 100, 128, 256])
+@pytest.mark.parametrize("k", [64, 1, 2, 3, 8, 32, 96, 100, 128, 256, 260, 512, 515])
 def test_spmm_matches_oracle_over_widths(gpu, oracle, dtype, k):
     A = gen.fixed_degree_random(4096 + 3, 32, seed=4004, dtype=dtype)
     B = gen.uniform_matrix(A.ncols, k, 4005).astype(dtype)
@@ -90,3 +92,70 @@ def test_batched_csrv_product_of_the_bspmm_example(gpu, oracle):
         torch.cuda.synchronize()
         assert np.allclose(gold, out.cpu().numpy())  # the example's acceptance check
         assert np.array_equal(out.cpu().numpy(), oracle.bspmm_csrv(pos, crd, values, V, m))  # same order: bit-exact
+
+
+def _banded(n, offsets, seed, dtype):
+    """Rows with one entry per in-range diagonal offset (a stencil's sparsity) and random values."""
+    rng = np.random.default_rng(seed)
+    diags = [rng.uniform(-1, 1, n - abs(o)) for o in offsets]
+    A = sp.diags(diags, offsets, shape=(n, n), format="csr")
+    A.sort_indices()
+    return gen.CSR(n, n, A.indptr.astype(np.int32), A.indices.astype(np.int32), A.data.astype(dtype))
+
+
+@pytest.mark.parametrize("dtype,k", [(np.float32, 64), (np.float32, 16), (np.float32, 256), (np.float64, 32),
+                                     (np.float64, 8), (np.float64, 128)])
+def test_planned_spmm_on_banded_matrices_through_every_kernel(gpu, oracle, dtype, k, monkeypatch):
+    # a 7-point stencil's pattern on 30 x 30 x 7 points: five of the seven diagonals lie inside the staged window
+    n = 30 * 30 * 7
+    A = _banded(n, [-900, -30, -1, 0, 1, 30, 900], 71, dtype)
+    plan = gpu.CsrPlan(A.nrows, A.ncols, dev(A.pos), dev(A.crd), value_bytes=np.dtype(dtype).itemsize)
+    near = plan.stats()["near_diagonal_fraction"]
+    want_near = [np.mean(np.abs(A.crd - np.repeat(np.arange(n), np.diff(A.pos))) <= h) for h in (32, 64, 128, 256)]
+    assert np.allclose(near, want_near, atol=1e-12)
+    B = gen.uniform_matrix(n, k, 72).astype(dtype)
+    C_in = gen.uniform_matrix(n, k, 73).astype(dtype)
+    _check(gpu, oracle, A, B, C_in, dtype, "banded k=%d planned" % k, plan=True)  # the plan picks group per row
+    # the same through both kernels explicitly: they must agree with the oracle on their own
+    for which in ("lds", "wave", "group"):
+        monkeypatch.setenv("LAPIS_HIP_SPMM_KERNEL", which)
+        _check(gpu, oracle, A, B, C_in, dtype, "banded k=%d forced %s" % (k, which), plan=True)
+    monkeypatch.delenv("LAPIS_HIP_SPMM_KERNEL")
+
+
+@pytest.mark.parametrize("which", ["lds", "group"])
+def test_staged_and_group_kernels_on_matrices_they_would_not_be_chosen_for(gpu, oracle, monkeypatch, which):
+    # forced onto random columns, ragged rows, blocks cut by the matrix end and a window cut by both ends of B
+    monkeypatch.setenv("LAPIS_HIP_SPMM_KERNEL", which)
+    for n, deg, k in ((5000, 9, 64), (700, 3, 32), (131, 5, 128)):
+        A = gen.fixed_degree_random(n, deg, seed=81 + n, dtype=np.float32)
+        B = gen.uniform_matrix(A.ncols, k, 82).astype(np.float32)
+        C_in = gen.uniform_matrix(A.nrows, k, 83).astype(np.float32)
+        _check(gpu, oracle, A, B, C_in, np.float32, "random n=%d k=%d forced lds" % (n, k), plan=True)
+    lengths = [0, 1, 63, 64, 65, 0, 0, 200, 3, 129, 0] * 30
+    A = _from_lengths(lengths, 330, 84, np.float64)
+    B = gen.uniform_matrix(330, 16, 85).astype(np.float64)
+    C_in = gen.uniform_matrix(len(lengths), 16, 86).astype(np.float64)
+    _check(gpu, oracle, A, B, C_in, np.float64, "ragged forced lds", plan=True)
+    # wide and short: more columns than rows, the window follows the row index
+    A = _from_lengths([7] * 600, 4000, 87, np.float32)
+    B = gen.uniform_matrix(A.ncols, 64, 88).astype(np.float32)
+    C_in = gen.uniform_matrix(A.nrows, 64, 89).astype(np.float32)
+    _check(gpu, oracle, A, B, C_in, np.float32, "wide forced lds", plan=True)
+    # tall: fewer columns than rows, the window of the last blocks lies past the end of B
+    A = _from_lengths([5] * 3000, 200, 90, np.float32)
+    B = gen.uniform_matrix(A.ncols, 64, 91).astype(np.float32)
+    C_in = gen.uniform_matrix(A.nrows, 64, 92).astype(np.float32)
+    _check(gpu, oracle, A, B, C_in, np.float32, "tall forced lds", plan=True)
+
+
+def test_planned_spmm_keeps_the_wave_kernel_for_random_columns_and_checks_the_plan(gpu, oracle):
+    A = gen.fixed_degree_random(20000, 32, seed=91, dtype=np.float32)
+    B = gen.uniform_matrix(A.ncols, 64, 92).astype(np.float32)
+    C_in = np.zeros((A.nrows, 64), np.float32)
+    plan = gpu.CsrPlan(A.nrows, A.ncols, dev(A.pos), dev(A.crd), value_bytes=4)
+    assert max(plan.stats()["near_diagonal_fraction"]) < 0.05
+    _check(gpu, oracle, A, B, C_in, np.float32, "random planned", plan=True)
+    with pytest.raises(gpu.LapisHipError) as e:  # a plan of another matrix
+        gpu.spmm(A.nrows, A.ncols, dev(A.pos), dev(A.crd), dev(A.val), dev(B), dev(C_in), plan=plan)
+    assert e.value.status_name == "LAPIS_HIP_ERR_PLAN_MISMATCH"
