@@ -52,8 +52,9 @@ def test_status_names_are_distinct():
 
 
 def test_stats_struct_matches_header_layout():
-    # 6 int64 + 3 double + int64 + 6 int32 = 104 bytes, no padding surprises
-    assert ctypes.sizeof(hip.CsrStats) == 6 * 8 + 3 * 8 + 8 + 6 * 4
+    # 6 int64 + 3 double + int64 + 6 int32 + 4 double = 136 bytes, no padding surprises
+    assert ctypes.sizeof(hip.CsrStats) == 6 * 8 + 3 * 8 + 8 + 6 * 4 + 4 * 8
+    assert hip.CsrStats.near_diagonal_fraction.offset == 104
 
 
 @pytest.mark.parametrize("dtype", [np.float64, np.float32, np.int32])
