@@ -225,7 +225,7 @@ __global__ __launch_bounds__(64 * WAVES) void spmv_nnzsplit_kernel(
   stage_products<T, CH, VEC, NT>(buf, lane, crd, val, x, e0, len, len);
   wave_lds_sync();
 
-  for (long long rb = r0; rb <= r1; rb += 64) {
+  for (long long rb = r0; rb <= r1;) {
     const long long r = rb + lane;
     int ps = 0, pe = 0;
     if (r <= r1) {
@@ -245,6 +245,22 @@ __global__ __launch_bounds__(64 * WAVES) void spmv_nnzsplit_kernel(
       else
         part_last[c] = acc;
     }
+    // Runs of empty rows must not cost a trip per 64 of them: after 64 rows without a
+    // single entry the next row that has one is found by bisection (positions are
+    // sorted), and rows that start at or behind the end of the chunk end the walk.
+    const int ps_first = __shfl(ps, 0, 64);
+    const int pe_last = __shfl(pe, 63, 64);
+    if (ps_first >= e1) break;
+    long long next = rb + 64;
+    if (next <= r1 && pe_last == ps_first) {
+      long long lo_r = next, hi_r = r1;  // first row in [next, r1] with pos[row + 1] > pe_last, else r1
+      while (lo_r < hi_r) {
+        const long long mid = (lo_r + hi_r) >> 1;
+        if (pos[mid + 1] > pe_last) hi_r = mid; else lo_r = mid + 1;
+      }
+      next = lo_r;
+    }
+    rb = next;
   }
 }
 

@@ -422,3 +422,52 @@ def test_analyze_builds_the_copy_only_where_it_is_recommended(gpu, oracle):
     plan = gpu.CsrPlan(L.nrows, L.ncols, lp, lc)
     plan.analyze(lc, lv)
     assert plan.stats()["kernel_name"] == "nnzsplit" and plan.stats()["colblock_layout_name"] is None
+
+
+@pytest.mark.parametrize("kernel", ["nnzsplit", "rowblock"])
+def test_long_runs_of_empty_rows(gpu, oracle, kernel):
+    # three million empty rows between the rows that hold the entries of one chunk, and again before the last row
+    rng = np.random.default_rng(5)
+    lengths = np.zeros(4_000_000, dtype=np.int64)
+    lengths[[0, 1, 2, 70, 3_000_000, 3_000_001, 3_999_999]] = [3, 600, 2, 90, 700, 5, 40]
+    lengths[rng.integers(3_000_002, 3_999_000, 50)] = rng.integers(1, 30, 50)
+    A = _from_lengths(lengths, 5000, 77, np.float64)
+    x = gen.uniform_vector(A.ncols, 78)
+    y_in = gen.uniform_vector(A.nrows, 79)
+    want = y_in.copy()
+    oracle.spmv(A.pos, A.crd, A.val, x, want)
+    scale = oracle.spmv_abs_scale(A.pos, A.crd, A.val, x, y_in)
+    pos, crd, val = dev(A.pos), dev(A.crd), dev(A.val)
+    plan = gpu.CsrPlan(A.nrows, A.ncols, pos, crd)
+    plan.set_kernel({"rowblock": 2, "nnzsplit": 3}[kernel])
+    y = dev(y_in)
+    gpu.spmv(plan, A.nrows, A.ncols, pos, crd, val, dev(x), y)
+    torch.cuda.synchronize()
+    assert_rows_close(y.cpu().numpy(), want, scale, np.float64, "empty runs/" + kernel)
+
+
+def test_config1_at_its_full_size(gpu, oracle):
+    # BASELINE config 1 itself: the 5-point Laplacian on the 256 x 256 grid (65 536 rows, 326 656 non-zeros)
+    A, x = gen.config1()
+    assert (A.nrows, A.nnz) == (65536, 326656)
+    want = np.zeros(A.nrows)
+    oracle.spmv(A.pos, A.crd, A.val, x, want)
+    scale = oracle.spmv_abs_scale(A.pos, A.crd, A.val, x)
+    pos, crd, val, dx = dev(A.pos), dev(A.crd), dev(A.val), dev(x)
+    for kernel in (0, 1, 2, 3):  # the plan's choice, then each CSR kernel family
+        plan = gpu.CsrPlan(A.nrows, A.ncols, pos, crd)
+        if kernel:
+            plan.set_kernel(kernel, 1 if kernel == 1 else 0)
+        y = torch.zeros(A.nrows, dtype=torch.float64, device="cuda")
+        gpu.spmv(plan, A.nrows, A.ncols, pos, crd, val, dx, y)
+        torch.cuda.synchronize()
+        got = y.cpu().numpy()
+        assert_rows_close(got, want, scale, np.float64, "config1/kernel %d" % kernel)
+        if kernel in (1, 2):  # one lane per row and the row-block kernel add in the oracle's order: bit for bit
+            assert np.array_equal(got, want)
+    # interior rows of a Laplacian annihilate the constant vector
+    ones = torch.ones(A.ncols, dtype=torch.float64, device="cuda")
+    y = torch.zeros(A.nrows, dtype=torch.float64, device="cuda")
+    gpu.spmv(gpu.CsrPlan(A.nrows, A.ncols, pos, crd), A.nrows, A.ncols, pos, crd, val, ones, y)
+    interior = np.diff(A.pos) == 5
+    assert np.all(y.cpu().numpy()[interior] == 0.0)
