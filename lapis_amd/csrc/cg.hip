@@ -24,6 +24,7 @@
 #include "blas1.hpp"
 #include "common.hpp"
 #include "plan.hpp"
+#include "rowsplit_fix.hpp"
 
 namespace lapis {
 
@@ -117,6 +118,60 @@ __global__ __launch_bounds__(256) void cg_pap_kernel(long long n, const double *
   CG_GRID_STRIDE(i, 2 * nv, n) acc = acc + p[i] * Ap[i];
   const double bsum = block_sum_256d(acc, lds4);
   if (threadIdx.x == 0) partials[blockIdx.x] = bsum;
+}
+
+// The same partials when Ap came from the row-split SpMV kernel with its fix-up left out:
+// a block takes `rows_per_block` consecutive rows (an even number, so the 128-bit accesses
+// stay aligned), first completes the rows of its range that are cut at chunk boundaries
+// (boundaries block_c[b] .. block_c[b+1]-1), then sums.  Only this block reads those rows
+// in this kernel, so a workgroup barrier orders the completion before the sum.
+template <int CH>
+__global__ __launch_bounds__(256) void cg_pap_fix_kernel(long long n, long long rows_per_block,
+                                                         const double *__restrict__ p, double *Ap,
+                                                         double *__restrict__ partials, int vec, int nchunks,
+                                                         const int *__restrict__ pos,
+                                                         const int *__restrict__ chunk_row,
+                                                         const double *__restrict__ part_first,
+                                                         const double *__restrict__ part_last,
+                                                         const int *__restrict__ block_c) {
+  __shared__ double lds4[4];
+  const int c0 = block_c[blockIdx.x], c1 = block_c[blockIdx.x + 1];
+  for (int base = c0; base < c1; base += 256) {
+    const long long c = (long long)base + threadIdx.x;
+    rowsplit_complete_row<double, CH>(c < c1 ? c : nchunks, nchunks, pos, chunk_row, part_first, part_last, Ap, 0);
+  }
+  __syncthreads();
+  const long long r0 = std::min(n, (long long)blockIdx.x * rows_per_block);
+  const long long r1 = std::min(n, r0 + rows_per_block);
+  double acc = 0.0;
+  if (vec) {
+    for (long long i = r0 / 2 + threadIdx.x; i < r1 / 2; i += 256) {
+      const v2d a = ld2(p, i), b = ld2(Ap, i);
+      acc = acc + a.x * b.x;
+      acc = acc + a.y * b.y;
+    }
+    if ((r1 & 1) && threadIdx.x == 0) acc = acc + p[r1 - 1] * Ap[r1 - 1];  // r1 is odd only where it is n
+  } else {
+    for (long long i = r0 + threadIdx.x; i < r1; i += 256) acc = acc + p[i] * Ap[i];
+  }
+  const double bsum = block_sum_256d(acc, lds4);
+  if (threadIdx.x == 0) partials[blockIdx.x] = bsum;
+}
+
+// block_c[b] = first chunk boundary c in [1, nchunks] whose row chunk_row[c] is at or behind
+// row b * rows_per_block (b = 0 .. blocks); chunk_row ascends and chunk_row[nchunks] is n.
+__global__ __launch_bounds__(256) void cg_fix_ranges_kernel(int blocks, long long n, long long rows_per_block,
+                                                            int nchunks, const int *__restrict__ chunk_row,
+                                                            int *__restrict__ block_c) {
+  const int b = blockIdx.x * 256 + threadIdx.x;
+  if (b > blocks) return;
+  const long long r = std::min(n, (long long)b * rows_per_block);
+  int lo = 1, hi = nchunks;
+  while (lo < hi) {
+    const int mid = lo + (hi - lo) / 2;
+    if (chunk_row[mid] >= r) hi = mid; else lo = mid + 1;
+  }
+  block_c[b] = lo;
 }
 
 // x += alpha p ; r -= alpha Ap ; block partials of r.r.   alpha = r.z / p.Ap with p.Ap
@@ -348,7 +403,7 @@ int pcg_run(lapis_hip_csr_plan *plan, int64_t n, const int32_t *pos, const int32
   double *tmp = mask ? work + 4 * stride : nullptr;
   const int divide = mask ? 1 : 0;
   PCG_TRY(hipMalloc(&state, sizeof(CgState)));
-  PCG_TRY(hipMalloc(&partials, sizeof(double) * 3 * kDotMaxBlocks));
+  PCG_TRY(hipMalloc(&partials, sizeof(double) * 3 * kDotMaxBlocks + sizeof(int) * (kDotMaxBlocks + 1)));
   CgState h{};
   h.maxiter = maxiter;
   h.tol = tol;
@@ -365,14 +420,14 @@ int pcg_run(lapis_hip_csr_plan *plan, int64_t n, const int32_t *pos, const int32
   hipLaunchKernelGGL(cg_init_scalar_kernel, dim3(1), dim3(256), 0, st, grid, partials, state);
   PCG_TRY(hipGetLastError());
   double *pap_partials = partials, *rr_partials = partials + kDotMaxBlocks, *rz_partials = partials + 2 * kDotMaxBlocks;
+  // rows per block of the p.Ap kernel that also completes the rows the row-split SpMV cuts (an even number)
+  int *block_c = reinterpret_cast<int *>(partials + 3 * kDotMaxBlocks);
+  const long long rows_per_block = ((((long long)n + grid - 1) / grid) + 1) & ~1LL;
+  bool ranges_ready = false;
 
   // The host looks at the device's `done` flag after each batch of iterations; a
   // batch queued past convergence costs launches only (its kernels return at once
   // or touch scratch vectors only).
-  struct Peek {
-    unsigned long long iter;
-    int done;
-  };
   uint64_t launched = 0;
   int batch = 1;
   while (!finished) {
@@ -385,6 +440,7 @@ int pcg_run(lapis_hip_csr_plan *plan, int64_t n, const int32_t *pos, const int32
                        (unsigned long long)launched);
     }
     for (int it = 0; it < todo; ++it) {
+      int deferred = 0;  // chunk length when the SpMV left its cut rows to the p.Ap kernel
       if (mask) {
         // plpt: tmp = mask*p ; Ap = A tmp ; Ap = (d*tmp - Ap)*mask
         PCG_RC(lapis_hip_mult_f64(n, p, mask, tmp, stream));
@@ -392,10 +448,31 @@ int pcg_run(lapis_hip_csr_plan *plan, int64_t n, const int32_t *pos, const int32
         hipLaunchKernelGGL(masked_combine_kernel, dim3(grid), dim3(256), 0, st, (long long)n, 0, dinv, tmp, mask, Ap);
       } else {
         // Ap = A p: the reference zero-fills Ap and accumulates (examples/pcg_solve.py:12-19)
-        PCG_RC(spmv_overwrite_f64(plan, n, n, pos, crd, val, p, Ap, stream));
+        PCG_RC(spmv_overwrite_f64(plan, n, n, pos, crd, val, p, Ap, stream, &deferred));
       }
       const unsigned long long iter = launched + (uint64_t)it + 1;  // the reference's counter for this pass
-      hipLaunchKernelGGL(cg_pap_kernel, dim3(grid), dim3(256), 0, st, (long long)n, p, Ap, pap_partials, vec);
+      if (deferred) {
+        if (!ranges_ready) {
+          hipLaunchKernelGGL(cg_fix_ranges_kernel, dim3((grid + 256) / 256), dim3(256), 0, st, grid, (long long)n,
+                             rows_per_block, plan->nchunks, (const int *)plan->chunk_row, block_c);
+          ranges_ready = true;
+        }
+#define PCG_PAP_FIX(CH)                                                                                              \
+  hipLaunchKernelGGL(cg_pap_fix_kernel<CH>, dim3(grid), dim3(256), 0, st, (long long)n, rows_per_block, p, Ap,       \
+                     pap_partials, vec, plan->nchunks, pos, (const int *)plan->chunk_row,                            \
+                     (const double *)plan->part_first, (const double *)plan->part_last, (const int *)block_c)
+        switch (deferred) {
+          case 512: PCG_PAP_FIX(512); break;
+          case 1024: PCG_PAP_FIX(1024); break;
+          case 2048: PCG_PAP_FIX(2048); break;
+          default:
+            cleanup();
+            return set_error(LAPIS_HIP_ERR_RUNTIME, "pcg: no p.Ap kernel for chunks of %d non-zeros", deferred);
+        }
+#undef PCG_PAP_FIX
+      } else {
+        hipLaunchKernelGGL(cg_pap_kernel, dim3(grid), dim3(256), 0, st, (long long)n, p, Ap, pap_partials, vec);
+      }
       hipLaunchKernelGGL(cg_update_xr_kernel, dim3(grid), dim3(256), 0, st, (long long)n, p, Ap, x, r, state, iter,
                          grid, pap_partials, rr_partials, vec);
       if (pre)

@@ -79,8 +79,9 @@ int sort_keys_with_perm(const unsigned long long *keys_in, int64_t nnz, int end_
 template <typename T>
 int gather_values(const unsigned *perm, const T *val, T *out, int64_t nnz, hipStream_t st);
 
-// y = A x without reading y; defined in spmv.hip.
+// y = A x without reading y; defined in spmv.hip.  A caller that passes `deferred_chunk` and gets a
+// non-zero chunk length back completes the rows cut at chunk boundaries itself (rowsplit_fix.hpp).
 int spmv_overwrite_f64(lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, const int32_t *pos,
                        const int32_t *crd, const double *val, const double *x, double *y,
-                       lapis_hip_stream_t stream);
+                       lapis_hip_stream_t stream, int *deferred_chunk = nullptr);
 }  // namespace lapis

@@ -12,6 +12,7 @@
 
 #include "common.hpp"
 #include "plan.hpp"
+#include "rowsplit_fix.hpp"
 
 namespace lapis {
 
@@ -264,46 +265,13 @@ __global__ __launch_bounds__(64 * WAVES) void spmv_nnzsplit_kernel(
   }
 }
 
-// One thread per chunk boundary c (1 <= c < nchunks).  The row cut by boundary c
-// is completed by the thread of the FIRST boundary that cuts it:
-//   y[r] += part_last[c-1] + part_first[c] + ... + part_first[c_last]
-// in that fixed order, so the result does not depend on scheduling.
+// One thread per chunk boundary c (1 <= c < nchunks); see rowsplit_complete_row.
 template <typename T, int CH>
 __global__ __launch_bounds__(256) void spmv_nnzsplit_fixup_kernel(
     int nchunks, const int *__restrict__ pos, const int *__restrict__ chunk_row,
     const T *__restrict__ part_first, const T *__restrict__ part_last, T *__restrict__ y, int accumulate) {
-  const int lane = threadIdx.x & 63;
   const long long c = (long long)blockIdx.x * 256 + threadIdx.x + 1;
-  bool owner = false;
-  int r = 0, cfirst = 0, clast = -1;
-  if (c < nchunks) {
-    r = chunk_row[c];
-    const long long ps = pos[r];
-    const long long b = c * CH;
-    if (ps < b && ps >= b - CH) {
-      owner = true;
-      cfirst = (int)c;
-      clast = (pos[r + 1] - 1) / CH;
-    }
-  }
-  const bool is_long = owner && (clast - cfirst) >= 16;
-  T total = T(0);
-  if (owner && !is_long) {
-    total = part_last[cfirst - 1];
-    for (int cc = cfirst; cc <= clast; ++cc) total = total + part_first[cc];
-  }
-  unsigned long long m = __ballot(is_long);
-  while (m) {
-    const int src = __builtin_ctzll(m);
-    m &= m - 1;
-    const int cs = __shfl(cfirst, src, 64);
-    const int cl = __shfl(clast, src, 64);
-    T part = T(0);
-    for (int cc = cs + lane; cc <= cl; cc += 64) part = part + part_first[cc];
-    part = group_sum<64>(part);
-    if (lane == src) total = part_last[cfirst - 1] + part;
-  }
-  if (owner) y[r] = accumulate ? total + y[r] : total;
+  rowsplit_complete_row<T, CH>(c, nchunks, pos, chunk_row, part_first, part_last, y, accumulate);
 }
 
 // ------------------------------------------------------------------------------
@@ -530,7 +498,7 @@ int launch_rowblock(int64_t nrows, int64_t nnz, const int *pos, const int *crd, 
 
 template <typename T, bool VEC, bool NT, int CH, int WPB>
 int launch_nnzsplit_cfg(const lapis_hip_csr_plan *p, const int *pos, const int *crd, const T *val, const T *x,
-                        T *y, hipStream_t st, int accumulate) {
+                        T *y, hipStream_t st, int accumulate, bool defer_fixup) {
   const int nchunks = p->nchunks;
   const int blocks = (int)ceil_div(nchunks, WPB);
   launch_timed(spmv_nnzsplit_kernel<T, CH, WPB, VEC, NT>, dim3(blocks), dim3(64 * WPB),
@@ -538,7 +506,7 @@ int launch_nnzsplit_cfg(const lapis_hip_csr_plan *p, const int *pos, const int *
                (const int *)p->chunk_row, static_cast<T *>(p->part_first), static_cast<T *>(p->part_last), accumulate,
                p->xcd_map);
   LAPIS_LAUNCH_CHECK();
-  if (nchunks > 1) {
+  if (nchunks > 1 && !defer_fixup) {
     const int fblocks = (int)ceil_div(nchunks - 1, 256);
     hipLaunchKernelGGL((spmv_nnzsplit_fixup_kernel<T, CH>), dim3(fblocks), dim3(256), 0, st, nchunks, pos,
                        p->chunk_row, static_cast<const T *>(p->part_first),
@@ -550,15 +518,15 @@ int launch_nnzsplit_cfg(const lapis_hip_csr_plan *p, const int *pos, const int *
 
 template <typename T, bool VEC, bool NT>
 int launch_nnzsplit(const lapis_hip_csr_plan *p, const int *pos, const int *crd, const T *val, const T *x,
-                    T *y, hipStream_t st, int accumulate = 1) {
+                    T *y, hipStream_t st, int accumulate = 1, bool defer_fixup = false) {
   switch (p->stats.chunk * 16 + p->waves_per_block) {
-    case 512 * 16 + 4: return launch_nnzsplit_cfg<T, VEC, NT, 512, 4>(p, pos, crd, val, x, y, st, accumulate);
-    case 512 * 16 + 8: return launch_nnzsplit_cfg<T, VEC, NT, 512, 8>(p, pos, crd, val, x, y, st, accumulate);
-    case 1024 * 16 + 2: return launch_nnzsplit_cfg<T, VEC, NT, 1024, 2>(p, pos, crd, val, x, y, st, accumulate);
-    case 1024 * 16 + 4: return launch_nnzsplit_cfg<T, VEC, NT, 1024, 4>(p, pos, crd, val, x, y, st, accumulate);
-    case 1024 * 16 + 8: return launch_nnzsplit_cfg<T, VEC, NT, 1024, 8>(p, pos, crd, val, x, y, st, accumulate);
-    case 2048 * 16 + 2: return launch_nnzsplit_cfg<T, VEC, NT, 2048, 2>(p, pos, crd, val, x, y, st, accumulate);
-    case 2048 * 16 + 4: return launch_nnzsplit_cfg<T, VEC, NT, 2048, 4>(p, pos, crd, val, x, y, st, accumulate);
+    case 512 * 16 + 4: return launch_nnzsplit_cfg<T, VEC, NT, 512, 4>(p, pos, crd, val, x, y, st, accumulate, defer_fixup);
+    case 512 * 16 + 8: return launch_nnzsplit_cfg<T, VEC, NT, 512, 8>(p, pos, crd, val, x, y, st, accumulate, defer_fixup);
+    case 1024 * 16 + 2: return launch_nnzsplit_cfg<T, VEC, NT, 1024, 2>(p, pos, crd, val, x, y, st, accumulate, defer_fixup);
+    case 1024 * 16 + 4: return launch_nnzsplit_cfg<T, VEC, NT, 1024, 4>(p, pos, crd, val, x, y, st, accumulate, defer_fixup);
+    case 1024 * 16 + 8: return launch_nnzsplit_cfg<T, VEC, NT, 1024, 8>(p, pos, crd, val, x, y, st, accumulate, defer_fixup);
+    case 2048 * 16 + 2: return launch_nnzsplit_cfg<T, VEC, NT, 2048, 2>(p, pos, crd, val, x, y, st, accumulate, defer_fixup);
+    case 2048 * 16 + 4: return launch_nnzsplit_cfg<T, VEC, NT, 2048, 4>(p, pos, crd, val, x, y, st, accumulate, defer_fixup);
     default:
       return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT, "spmv: no row-split kernel for %d non-zeros per wavefront, %d wavefronts per block",
                        p->stats.chunk, p->waves_per_block);
@@ -637,16 +605,25 @@ int spmv_impl(lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, const int3
 namespace lapis {
 // y = A x (y is not read).  The row-split kernel writes every non-empty row itself;
 // any other case zero-fills y and accumulates.
+//
+// With `deferred_chunk` the caller offers to complete the rows cut at chunk boundaries
+// itself (rowsplit_complete_row over boundaries 1..nchunks-1 with the plan's chunk_row,
+// part_first and part_last, accumulate = 0): when the row-split kernel runs, its fix-up
+// launch is left out and *deferred_chunk is the chunk length, otherwise it is 0 and y is complete.
 int spmv_overwrite_f64(lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, const int32_t *pos,
                        const int32_t *crd, const double *val, const double *x, double *y,
-                       lapis_hip_stream_t stream) {
+                       lapis_hip_stream_t stream, int *deferred_chunk) {
+  if (deferred_chunk) *deferred_chunk = 0;
   if (plan && plan->stats.kernel == LAPIS_HIP_SPMV_NNZSPLIT && plan->stats.empty_rows == 0 && plan->stats.nnz > 0 &&
       plan->stats.nrows == nrows && plan->stats.ncols == ncols && plan->pos == pos && aligned16(crd) &&
       aligned16(val)) {
     LAPIS_CHECK_INIT();
     hipStream_t st = as_stream(stream);
-    return plan->nontemporal ? launch_nnzsplit<double, true, true>(plan, pos, crd, val, x, y, st, 0)
-                             : launch_nnzsplit<double, true, false>(plan, pos, crd, val, x, y, st, 0);
+    const bool defer = deferred_chunk && plan->nchunks > 1;
+    const int rc = plan->nontemporal ? launch_nnzsplit<double, true, true>(plan, pos, crd, val, x, y, st, 0, defer)
+                                     : launch_nnzsplit<double, true, false>(plan, pos, crd, val, x, y, st, 0, defer);
+    if (rc == LAPIS_HIP_OK && defer) *deferred_chunk = plan->stats.chunk;
+    return rc;
   }
   const int rc = lapis_hip_fill_f64(nrows, 0.0, y, stream);
   if (rc != LAPIS_HIP_OK) return rc;
