@@ -201,6 +201,16 @@ def run_spmv(args, cfg):
     kt = hip.kernel_timing_stop()
     bytes_step = A.spmv_bytes()
     ms = elapsed / args.steps * 1e3
+    update_ms = None
+    if stats["kernel_name"] == "colblock":
+        # what new values of the same structure cost: one gather pass through the kept permutation
+        plan.update_values(val)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(5):
+            plan.update_values(val)
+        torch.cuda.synchronize()
+        update_ms = (time.perf_counter() - t0) / 5 * 1e3
     family = "colgroup" if stats["colblock_layout_name"] == "group" else stats["kernel_name"]
     kernel_name = "spmv_%s_kernel<%s>" % (family, "double" if dtype == np.float64 else "float")
     achieved = bytes_step / (kt["mean_ms"] * 1e-3) / 1e9
@@ -216,7 +226,7 @@ def run_spmv(args, cfg):
                    "colblock_layout": stats["colblock_layout_name"],
                    "width": stats["width"], "chunk": stats["chunk"],
                    "reference_vector_length": stats["reference_vector_length"], "plan_ms": plan_ms,
-                   "csr_kernel_ms_per_call": csr_ms,
+                   "csr_kernel_ms_per_call": csr_ms, "colblock_update_values_ms": update_ms,
                    # calls of this matrix after which building the copy (outside the timed region) has paid back
                    "break_even_calls": (build_ms / (csr_ms - ms) if build_ms and csr_ms and csr_ms > ms else None)},
         "pct_of_hbm_peak": 100.0 * bytes_step / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
