@@ -14,10 +14,18 @@ computations the prebuilt gfx950 module implements (lapis_amd/catalogue.py).  A 
 of WHAT it computes: ``@matvec`` doing ``linalg.matvec`` on a CSR operand binds to the SpMV entry point
 under its own name, while a ``@spmv`` that multiplies by the transpose, or takes a CSC operand, is
 refused with the reference's message for a failed lowering.
+
+A module that is already lowered to loops binds too: a function whose one `scf.parallel` nest is the CSR
+SpMV nest the sparsifier produces (lapis_amd/loop_mapping.py decides the Kokkos level of every loop by the
+rules of the reference's loop-mapping pass and recognises that nest) is bound to the SpMV entry point, with
+its memref arguments routed by the ROLE each plays in the nest (y, positions, coordinates, values, x).
 """
 import os
 
+import re
+
 from . import catalogue as _catalogue
+from . import loop_mapping as _lm
 from . import mlir_text as _mt
 from . import module as _module
 
@@ -41,6 +49,16 @@ def _public_functions(text):
     """(name, argument kinds, has a result) of the module's public functions."""
     c = _mt.Canonicalizer(text)
     return [(f.name, c.signature(f)[0], bool(f.results)) for f in c.public()]
+
+
+def _spmv_by_role(mod, order):
+    """Method for a loop-level SpMV function: memref arguments in the function's own order, y updated in place."""
+    def method(*args):
+        if len(args) != 5:
+            raise TypeError("expected 5 memref arguments, got %d" % len(args))
+        y, pos, crd, val, x = (args[order[r]] for r in ("y", "pos", "crd", "val", "x"))
+        mod.spmv(pos, crd, val, ((len(y), len(x)), (len(pos), len(crd), len(val))), x, y)
+    return method
 
 
 class KokkosBackend:
@@ -70,6 +88,7 @@ class KokkosBackend:
             raise Exception(_LOWERING_FAILED)
         bound = {}
         self.unbound = []
+        self.loop_mapping = {}   # function name -> loop_mapping.NestMapping of a function bound at loop level
         for f in public:
             method = "lapis_main" if f.name == "main" else f.name
             kinds, results = c.signature(f)
@@ -80,6 +99,10 @@ class KokkosBackend:
             except _mt.ParseError as e:
                 raise Exception(_LOWERING_FAILED + "\n@%s could not be read: %s" % (f.name, e))
             entry = _forms().get(form)
+            if entry is None:
+                entry, why_not = self._loop_level_entry(f)
+                if entry is None and why_not:
+                    raise Exception("%s\nfunction @%s: %s" % (_LOWERING_FAILED, f.name, why_not))
             if entry is None:
                 if not results:
                     # a helper that returns nothing (the sparse_tensor.print wrapper of examples/bspmm.py:54-58):
@@ -97,6 +120,41 @@ class KokkosBackend:
             bound[method] = entry
         return bound
 
+    def _loop_level_entry(self, f):
+        """(("loops:spmv", {role: argument index}), None) when @f is one CSR SpMV loop nest over 32-bit
+        positions and coordinates and nothing else; (None, reason) for any other function made of loops;
+        (None, None) for a function without `scf.parallel`."""
+        if "scf.parallel" not in f.body:
+            return None, None
+        try:
+            nests = _lm.map_function_body(f.body, hip_kernels=True)
+        except (_mt.ParseError, AttributeError, ValueError) as e:
+            return None, "its loops could not be read: %s" % e
+        described = "; ".join("%s nest of depth %d" % (n.space, n.depth) for n in nests)
+        if len(nests) != 1 or not nests[0].csr_spmv or f.results:
+            return None, ("its loops (%s) are not the one CSR SpMV nest y[i] += sum_j val[pos[i]+j] * x[crd[pos[i]+j]] "
+                          "the gfx950 module implements" % described)
+        roles = nests[0].csr_spmv
+        stmts, _ = _mt.read_region(f.body)
+        if any(s.op not in ("arith.constant", "memref.dim", "scf.parallel", "return", "func.return") for s in stmts):
+            return None, "it does more than the one CSR SpMV nest"
+        names = [nm for nm, _ in f.args]
+        types = dict(f.args)
+        order = {}
+        for role in ("y", "pos", "crd", "val", "x"):
+            if roles[role] not in names:
+                return None, "the %s buffer of its SpMV nest is not a function argument" % role
+            order[role] = names.index(roles[role])
+            want = "i32" if role in ("pos", "crd") else roles["elem"]
+            have = types[roles[role]].replace(" ", "")
+            if not re.match(r"memref<\?x%s>$" % want, have):
+                return None, ("the %s buffer of its SpMV nest is %s; the module implements 32-bit positions and "
+                              "coordinates and contiguous one-dimensional memref<?x%s>" % (role, have, want))
+        if len(set(order.values())) != 5:
+            return None, "two buffers of its SpMV nest are the same argument"
+        self.loop_mapping[f.name] = nests[0]
+        return ("loops:spmv", order), None
+
     def compile(self, module):
         moduleText = str(module)
         if self.dump_mlir:
@@ -106,7 +164,9 @@ class KokkosBackend:
         mod = _module.LAPISModule()
         mod.bound_functions = sorted(bound)
         for method, entry in bound.items():
-            if method != entry:
+            if isinstance(entry, tuple):
+                setattr(mod, method, _spmv_by_role(mod, entry[1]))
+            elif method != entry:
                 setattr(mod, method, getattr(mod, entry))  # the function's own name, the entry its body calls for
         for name in self.unbound:
             def _not_implemented(*args, _name=name, **kwargs):

@@ -4,6 +4,7 @@ import re
 
 import pytest
 
+import loop_nests
 import modules_mlir as M
 from lapis_amd import mlir_text
 from lapis_amd.KokkosBackend import KokkosBackend, _public_functions
@@ -94,3 +95,28 @@ def test_constructor_mirrors_the_reference():
     b = KokkosBackend(decompose_tensors=True, parallel_strategy="dense-outer-loop", index_instance=2, num_instances=3)
     assert b.package_name == "lapis_package_2" and b.parallel_strategy == "dense-outer-loop"
     assert KokkosBackend().package_name == "lapis_package"
+
+
+def test_a_module_already_lowered_to_loops_binds_by_the_roles_in_its_nest():
+    b = KokkosBackend(decompose_tensors=True)
+    bound = b.bind(loop_nests.spmv_i32("f64", name="apply"))
+    # arguments of @apply are (vals, x, rowptr, y, colidx): routed by what the nest does with them
+    assert bound == {"apply": ("loops:spmv", {"y": 3, "pos": 2, "crd": 4, "val": 0, "x": 1})}
+    m = b.loop_mapping["apply"]
+    assert m.depth == 2 and m.space == "device" and m.vector_length_hint is None  # the library's plan decides
+
+
+def test_loop_level_functions_that_are_not_the_spmv_nest_are_refused_with_the_reason():
+    b = KokkosBackend(decompose_tensors=True)
+    with pytest.raises(Exception, match=r"Lowering to Kokkos dialect failed.[\s\S]*memref<\?xindex>"):
+        b.bind(loop_nests.SPMV_INDEX)          # 64-bit positions
+    with pytest.raises(Exception, match=r"Lowering to Kokkos dialect failed.[\s\S]*depth 4"):
+        b.bind(loop_nests.DEEP4)
+    text = loop_nests.spmv_i32("f64").replace("arith.addf %rhs, %lhs", "arith.maximumf %rhs, %lhs")
+    with pytest.raises(Exception, match=r"not the one CSR SpMV nest"):
+        b.bind(text)
+    # the nest plus anything else in the function is not bound either
+    text = loop_nests.spmv_i32("f64").replace("    return\n", "    memref.store %x0, %y[%zero] : memref<?xf64>\n    return\n").replace(
+        "%rows = memref.dim", "%x0 = memref.load %x[%zero] : memref<?xf64>\n    %rows = memref.dim")
+    with pytest.raises(Exception, match=r"does more than"):
+        b.bind(text)

@@ -186,6 +186,30 @@ def test_compile_binds_spmv_by_its_body_and_reproduces_the_literal_answer(gpu, g
         backend.compile(M.SPMV_TRANSPOSED)
 
 
+def test_compile_binds_a_loop_level_spmv_and_routes_its_buffers_by_role(gpu, golden, oracle):
+    import loop_nests
+    from lapis_amd import KokkosBackend
+    g = golden["spmv_noalloc"]
+    rowptrs, colinds = np.array(g["pos"], np.int32), np.array(g["crd"], np.int32)
+    backend = KokkosBackend.KokkosBackend(decompose_tensors=True)
+    for elem, dtype, tol in (("f64", np.float64, 1e-14), ("f32", np.float32, 1e-6)):
+        module_kokkos = backend.compile(loop_nests.spmv_i32(elem, name="apply"))
+        values = np.array(g["val"], dtype)
+        y = np.zeros(5, dtype)
+        # @apply(vals, x, rowptr, y, colidx)
+        module_kokkos.apply(values, np.ones(5, dtype), rowptrs, y, colinds)
+        assert np.allclose(y, [1.1, 2.2, -19, -1, 0], rtol=tol, atol=tol)  # examples/spmv_noalloc.py:31
+        module_kokkos.apply(values, np.ones(5, dtype), rowptrs, y, colinds)  # the nest starts from y[i]: accumulates
+        assert np.allclose(y, 2 * np.array([1.1, 2.2, -19, -1, 0]), rtol=tol, atol=tol)
+    # a larger matrix against the oracle
+    A, x = gen.laplace2d(48), gen.uniform_vector(48 * 48, 5)
+    y = np.zeros(A.nrows)
+    backend.compile(loop_nests.spmv_i32("f64", name="apply")).apply(A.val, x, A.pos, y, A.crd)
+    want = np.zeros(A.nrows)
+    oracle.spmv(A.pos, A.crd, A.val, x, want)
+    assert np.allclose(y, want, rtol=1e-13, atol=1e-13)
+
+
 def test_compile_binds_pcg_and_matches_scipy_on_nos4(gpu):
     import modules_mlir as M
     from lapis_amd import KokkosBackend
