@@ -522,6 +522,7 @@ extern "C" int lapis_hip_csr_plan_update_values(lapis_hip_csr_plan *plan, const 
   if (value_bytes != plan->colblock_value_bytes)
     return set_error(LAPIS_HIP_ERR_PLAN_MISMATCH, "csr_plan_update_values: the copy holds %d-byte values, called with %d",
                      plan->colblock_value_bytes, value_bytes);
+  LAPIS_REQUIRE(plan->colblock_perm, "csr_plan_update_values: the copy was built without its permutation");
   hipStream_t st = as_stream(stream);
   const int rc = value_bytes == 8
                      ? gather_values<double>(plan->colblock_perm, static_cast<const double *>(val),
