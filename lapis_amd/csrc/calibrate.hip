@@ -12,6 +12,7 @@
 // every CU could keep a fixed number of line requests in flight whatever they are.
 // bench.py turns the two rates into the floor of the column-blocked SpMV kernels.
 #include <algorithm>
+#include <cstdlib>
 
 #include "common.hpp"
 
@@ -27,7 +28,31 @@ __device__ __forceinline__ unsigned mix32(unsigned a) {
   return a;
 }
 
-template <int THREADS, int GPT, int SB, bool GATHER>
+// GPT = 4 gathers with a chosen cache policy on the load (gfx950 `sc0`, `sc1`, `nt` bits): the probe for
+// whether a policy changes the rate at which L2 serves line requests.  It does not (256-269 G lines/s for
+// every combination, 4- and 8-byte elements alike), which is why the SpMV kernels use plain loads.
+template <int POLICY>
+__device__ __forceinline__ void gather4(const double *const (&p)[4], double (&g)[4]) {
+  if (POLICY == 0) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) g[j] = *p[j];
+    return;
+  }
+#define LAPIS_GATHER4(BITS)                                                                                        \
+  asm volatile("global_load_dwordx2 %0, %4, off " BITS "\n global_load_dwordx2 %1, %5, off " BITS                  \
+               "\n global_load_dwordx2 %2, %6, off " BITS "\n global_load_dwordx2 %3, %7, off " BITS               \
+               "\n s_waitcnt vmcnt(0)"                                                                             \
+               : "=&v"(g[0]), "=&v"(g[1]), "=&v"(g[2]), "=&v"(g[3])                                                \
+               : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3])                                                        \
+               : "memory")
+  if (POLICY == 1) LAPIS_GATHER4("nt");
+  if (POLICY == 2) LAPIS_GATHER4("sc0");
+  if (POLICY == 3) LAPIS_GATHER4("sc1");
+  if (POLICY == 4) LAPIS_GATHER4("sc0 sc1");
+#undef LAPIS_GATHER4
+}
+
+template <int THREADS, int GPT, int SB, bool GATHER, int POLICY>
 __global__ __launch_bounds__(THREADS) void calibrate_kernel(const v2d *__restrict__ stream, long long vecs_per_group,
                                                             const double *__restrict__ x, unsigned window_lines,
                                                             int share_log2, int steps, double *__restrict__ sink) {
@@ -43,12 +68,15 @@ __global__ __launch_bounds__(THREADS) void calibrate_kernel(const v2d *__restric
       for (int j = 0; j < SB; ++j) sv[j] = load_stream(sp + ((long long)s * SB + j) * THREADS + tid);
     }
     if (GATHER) {
+      static_assert(GPT == 4, "gather4 takes four addresses");
+      const double *gp[GPT];
 #pragma unroll
       for (int j = 0; j < GPT; ++j) {
         const unsigned line =
             mix32((wave * 4099u + (unsigned)s) * 64u * GPT + j * 64u + (lane >> share_log2)) % window_lines;
-        g[j] = x[(size_t)line * 16 + (lane & 15)];
+        gp[j] = x + (size_t)line * 16 + (lane & 15);
       }
+      gather4<POLICY>(gp, g);
 #pragma unroll
       for (int j = 0; j < GPT; ++j) acc += g[j];
     }
@@ -77,9 +105,25 @@ int run(const double *x, int64_t window_bytes, int share_log2, const void *strea
   LAPIS_HIP_TRY(hipEventCreate(&e1));
   float best = 0.f;
   hipError_t err = hipSuccess;
+  // LAPIS_HIP_CALIBRATE_POLICY = 1 (nt), 2 (sc0), 3 (sc1), 4 (sc0 sc1): cache policy of the gathers
+  const char *pol = GATHER ? getenv("LAPIS_HIP_CALIBRATE_POLICY") : nullptr;
+  const int policy = pol ? atoi(pol) : 0;
+  if (policy < 0 || policy > 4)
+    return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT, "calibrate_gather: LAPIS_HIP_CALIBRATE_POLICY must be 0..4, got %d", policy);
   for (int rep = 0; rep < 6 && err == hipSuccess; ++rep) {
-    hipExtLaunchKernelGGL((calibrate_kernel<THREADS, GPT, SB, GATHER>), dim3(groups), dim3(THREADS), 0, st, e0, e1, 0,
-                          static_cast<const v2d *>(stream), vecs_per_group, x, window_lines, share_log2, steps, sink);
+    const dim3 grid(groups), block(THREADS);
+    const v2d *sv = static_cast<const v2d *>(stream);
+#define LAPIS_CAL_LAUNCH(P)                                                                                       \
+  hipExtLaunchKernelGGL((calibrate_kernel<THREADS, GPT, SB, GATHER, P>), grid, block, 0, st, e0, e1, 0, sv,      \
+                        vecs_per_group, x, window_lines, share_log2, steps, sink)
+    switch (policy) {
+      case 1: LAPIS_CAL_LAUNCH(1); break;
+      case 2: LAPIS_CAL_LAUNCH(2); break;
+      case 3: LAPIS_CAL_LAUNCH(3); break;
+      case 4: LAPIS_CAL_LAUNCH(4); break;
+      default: LAPIS_CAL_LAUNCH(0); break;
+    }
+#undef LAPIS_CAL_LAUNCH
     err = hipGetLastError();
     if (err == hipSuccess) err = hipEventSynchronize(e1);
     float ms = 0.f;
