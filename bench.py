@@ -372,8 +372,7 @@ def run_spmm(args):
                    "near_diagonal_fraction": stats["near_diagonal_fraction"], "mean_row_len": stats["mean_row_len"]},
         "pct_of_hbm_peak": 100.0 * bytes_step / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "gflops": 2.0 * A.nnz * k / (ms * 1e-3) / 1e9,
-        "roofline": {"bound": "hbm", "kernel": "spmm kernel chosen by the plan (wave-per-row or LDS-staged row block)",
-                     "achieved": achieved,
+        "roofline": {"bound": "hbm", "kernel": "%s<float>" % hip.spmm_last_kernel(), "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": traffic_from_profiles("spmm_config4", kt["mean_ms"])
                      if not args.workload and k == 64 else None, "kernel_ms_mean": kt["mean_ms"],

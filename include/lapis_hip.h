@@ -256,6 +256,12 @@ int lapis_hip_spmm_csr_f64_i32_plan(const lapis_hip_csr_plan *plan, int64_t nrow
                                     const int32_t *pos, const int32_t *crd, const double *val, const double *B,
                                     int64_t ldb, double *C, int64_t ldc, lapis_hip_stream_t stream);
 
+/* Name of the kernel the calling thread's last SpMM call launched ("spmm_wave_row_kernel",
+ * "spmm_group_row_kernel", "spmm_rowblock_lds_kernel"; "" before the first call): benchmark lines name the
+ * kernel they timed with it.  No counterpart in the reference, whose loop mapping is fixed when the module
+ * is compiled (Pipelines/Passes.h:41-56). */
+const char *lapis_hip_spmm_last_kernel(void);
+
 /* Batched CSRV product of examples/bspmm.py:22-50 (out(n1,dh,nh) += A(n1,n2,nh) * V(n2,dh,nh)):
  * A is CSR over (n1, n2), each non-zero carries nh values (val has nnz*nh entries). */
 int lapis_hip_bspmm_csrv_f32_i32(int64_t n1, int64_t n2, int64_t dh, int64_t nh, const int32_t *pos,

@@ -334,6 +334,9 @@ int launch_rowblock_lds(int64_t nrows, int64_t ncols, int rb, int halo, const in
   return LAPIS_HIP_OK;
 }
 
+// name of the kernel the calling thread's last SpMM ran (lapis_hip_spmm_last_kernel)
+static thread_local const char *g_last_spmm_kernel = "";
+
 template <typename T>
 int spmm_impl(const char *what, const lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, int64_t k,
               const int32_t *pos, const int32_t *crd, const T *val, const T *B, int64_t ldb, T *C, int64_t ldc,
@@ -385,6 +388,7 @@ int spmm_impl(const char *what, const lapis_hip_csr_plan *plan, int64_t nrows, i
     if (use_group) use_lds = false;
   }
   if (use_group && !use_lds) {
+    g_last_spmm_kernel = "spmm_group_row_kernel";
     switch (lpr) {
       case 1: launch_group_row<T, 1>(nrows, pos, crd, val, B, ldb, C, ldc, st); break;
       case 2: launch_group_row<T, 2>(nrows, pos, crd, val, B, ldb, C, ldc, st); break;
@@ -397,6 +401,7 @@ int spmm_impl(const char *what, const lapis_hip_csr_plan *plan, int64_t nrows, i
     return LAPIS_HIP_OK;
   }
   if (use_lds) {
+    g_last_spmm_kernel = "spmm_rowblock_lds_kernel";
     switch (lpr) {
       case 4: return launch_rowblock_lds<T, 4>(nrows, ncols, rb, halo, pos, crd, val, B, ldb, C, ldc, st);
       case 8: return launch_rowblock_lds<T, 8>(nrows, ncols, rb, halo, pos, crd, val, B, ldb, C, ldc, st);
@@ -405,6 +410,7 @@ int spmm_impl(const char *what, const lapis_hip_csr_plan *plan, int64_t nrows, i
       default: return launch_rowblock_lds<T, 64>(nrows, ncols, rb, halo, pos, crd, val, B, ldb, C, ldc, st);
     }
   }
+  g_last_spmm_kernel = "spmm_wave_row_kernel";
   if (vec)
     launch_wave_row_any<T, true>(nrows, k, pos, crd, val, B, ldb, C, ldc, st);
   else
@@ -416,6 +422,8 @@ int spmm_impl(const char *what, const lapis_hip_csr_plan *plan, int64_t nrows, i
 }  // namespace lapis
 
 using namespace lapis;
+
+extern "C" const char *lapis_hip_spmm_last_kernel(void) { return g_last_spmm_kernel; }
 
 extern "C" int lapis_hip_spmm_csr_f32_i32(int64_t nrows, int64_t ncols, int64_t k, const int32_t *pos,
                                           const int32_t *crd, const float *val, const float *B, int64_t ldb,

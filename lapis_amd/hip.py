@@ -86,7 +86,8 @@ _SIGNATURES = {
 }
 
 # every symbol include/lapis_hip.h declares
-EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + ["lapis_hip_last_error", "lapis_hip_status_name"])
+EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + ["lapis_hip_last_error", "lapis_hip_status_name",
+                                             "lapis_hip_spmm_last_kernel"])
 
 _lib = None
 
@@ -106,6 +107,7 @@ def load(path=None):
         fn.argtypes = argtypes
         fn.restype = _int
     lib.lapis_hip_last_error.restype = ctypes.c_char_p
+    lib.lapis_hip_spmm_last_kernel.restype = ctypes.c_char_p
     lib.lapis_hip_status_name.restype = ctypes.c_char_p
     lib.lapis_hip_status_name.argtypes = [_int]
     _lib = lib
@@ -250,6 +252,11 @@ def spmm(nrows, ncols, pos, crd, val, B, C, stream=None, plan=None):
     check(fn(nrows, ncols, k, _ptr(pos), _ptr(crd), _ptr(val), _ptr(B), int(B.stride(0)), _ptr(C), int(C.stride(0)),
              _stream(stream)))
     return C
+
+
+def spmm_last_kernel():
+    """Name of the kernel this thread's last ``spmm`` call launched."""
+    return init().lapis_hip_spmm_last_kernel().decode()
 
 
 def dot(x, y, result, init_value=0.0, stream=None):

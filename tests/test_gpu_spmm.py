@@ -116,10 +116,16 @@ def test_planned_spmm_on_banded_matrices_through_every_kernel(gpu, oracle, dtype
     B = gen.uniform_matrix(n, k, 72).astype(dtype)
     C_in = gen.uniform_matrix(n, k, 73).astype(dtype)
     _check(gpu, oracle, A, B, C_in, dtype, "banded k=%d planned" % k, plan=True)  # the plan picks group per row
+    lanes_per_row = k * np.dtype(dtype).itemsize // 16
+    group_fits = lanes_per_row <= 32  # a row of B wider than half a wavefront leaves no room for a second group
+    assert gpu.spmm_last_kernel() == ("spmm_group_row_kernel" if group_fits else "spmm_wave_row_kernel")
     # the same through both kernels explicitly: they must agree with the oracle on their own
     for which in ("lds", "wave", "group"):
         monkeypatch.setenv("LAPIS_HIP_SPMM_KERNEL", which)
         _check(gpu, oracle, A, B, C_in, dtype, "banded k=%d forced %s" % (k, which), plan=True)
+        want = {"lds": "spmm_rowblock_lds_kernel", "wave": "spmm_wave_row_kernel",
+                "group": "spmm_group_row_kernel" if group_fits else "spmm_wave_row_kernel"}[which]
+        assert gpu.spmm_last_kernel() == want
     monkeypatch.delenv("LAPIS_HIP_SPMM_KERNEL")
 
 
