@@ -63,6 +63,8 @@ int lapis_hip_stream_synchronize(lapis_hip_stream_t stream);
  * in milliseconds (any output may be NULL). */
 int lapis_hip_kernel_timing_start(int capacity);
 int lapis_hip_kernel_timing_stop(int *count, double *mean_ms, double *min_ms, double *max_ms);
+/* Median, in milliseconds, of the launches the last lapis_hip_kernel_timing_stop read (0 before the first). */
+double lapis_hip_kernel_timing_median_ms(void);
 
 /* Measurement only (`bench.py --calibrate-gather`): one launch in the shape of the
  * column-blocked SpMV kernels -- one workgroup of 512 threads per compute unit,

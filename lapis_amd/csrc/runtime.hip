@@ -84,6 +84,8 @@ extern "C" int lapis_hip_finalize(void) {
   return LAPIS_HIP_OK;
 }
 
+static double g_timing_median = 0.0;  // of the launches the last kernel_timing_stop read
+
 extern "C" int lapis_hip_kernel_timing_start(int capacity) {
   LAPIS_CHECK_INIT();
   LAPIS_REQUIRE(capacity > 0 && capacity <= (1 << 20), "kernel_timing_start: capacity %d outside [1, 2^20]", capacity);
@@ -110,10 +112,12 @@ extern "C" int lapis_hip_kernel_timing_stop(int *count, double *mean_ms, double 
   hipError_t err = hipDeviceSynchronize();
   double sum = 0.0, mn = 0.0, mx = 0.0;
   int n = 0;
+  std::vector<float> all;
   for (int i = 0; err == hipSuccess && i < g_timing_used; ++i) {
     float ms = 0.f;
     err = hipEventElapsedTime(&ms, g_timing_events[2 * (size_t)i], g_timing_events[2 * (size_t)i + 1]);
     if (err != hipSuccess) break;
+    all.push_back(ms);
     sum += ms;
     mn = (n == 0) ? ms : std::min<double>(mn, ms);
     mx = (n == 0) ? ms : std::max<double>(mx, ms);
@@ -122,11 +126,21 @@ extern "C" int lapis_hip_kernel_timing_stop(int *count, double *mean_ms, double 
   timing_release();
   if (err != hipSuccess)
     return set_error(LAPIS_HIP_ERR_RUNTIME, "kernel_timing_stop: %s", hipGetErrorString(err));
+  g_timing_median = 0.0;
+  if (n) {
+    std::sort(all.begin(), all.end());
+    g_timing_median = (n & 1) ? all[n / 2] : 0.5 * ((double)all[n / 2 - 1] + all[n / 2]);
+  }
   if (count) *count = n;
   if (mean_ms) *mean_ms = n ? sum / n : 0.0;
   if (min_ms) *min_ms = mn;
   if (max_ms) *max_ms = mx;
   return LAPIS_HIP_OK;
+}
+
+extern "C" double lapis_hip_kernel_timing_median_ms(void) {
+  std::lock_guard<std::mutex> lock(g_timing_mutex);
+  return g_timing_median;
 }
 
 extern "C" const char *lapis_hip_last_error(void) { return g_error; }

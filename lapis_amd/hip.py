@@ -87,7 +87,7 @@ _SIGNATURES = {
 
 # every symbol include/lapis_hip.h declares
 EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + ["lapis_hip_last_error", "lapis_hip_status_name",
-                                             "lapis_hip_spmm_last_kernel"])
+                                             "lapis_hip_spmm_last_kernel", "lapis_hip_kernel_timing_median_ms"])
 
 _lib = None
 
@@ -108,6 +108,8 @@ def load(path=None):
         fn.restype = _int
     lib.lapis_hip_last_error.restype = ctypes.c_char_p
     lib.lapis_hip_spmm_last_kernel.restype = ctypes.c_char_p
+    lib.lapis_hip_kernel_timing_median_ms.restype = _dbl
+    lib.lapis_hip_kernel_timing_median_ms.argtypes = []
     lib.lapis_hip_status_name.restype = ctypes.c_char_p
     lib.lapis_hip_status_name.argtypes = [_int]
     _lib = lib
@@ -156,10 +158,12 @@ def kernel_timing_start(capacity):
 
 
 def kernel_timing_stop():
-    """-> dict(count, mean_ms, min_ms, max_ms) of the launches timed since the start call."""
+    """-> dict(count, mean_ms, median_ms, min_ms, max_ms) of the launches timed since the start call."""
     n, mean, mn, mx = _int(0), _dbl(0), _dbl(0), _dbl(0)
-    check(init().lapis_hip_kernel_timing_stop(ctypes.byref(n), ctypes.byref(mean), ctypes.byref(mn), ctypes.byref(mx)))
-    return {"count": n.value, "mean_ms": mean.value, "min_ms": mn.value, "max_ms": mx.value}
+    lib = init()
+    check(lib.lapis_hip_kernel_timing_stop(ctypes.byref(n), ctypes.byref(mean), ctypes.byref(mn), ctypes.byref(mx)))
+    return {"count": n.value, "mean_ms": mean.value, "median_ms": lib.lapis_hip_kernel_timing_median_ms(),
+            "min_ms": mn.value, "max_ms": mx.value}
 
 
 COLBLOCK_LAYOUTS = {"auto": 0, "wave": 1, "group": 2}

@@ -471,3 +471,20 @@ def test_config1_at_its_full_size(gpu, oracle):
     gpu.spmv(gpu.CsrPlan(A.nrows, A.ncols, pos, crd), A.nrows, A.ncols, pos, crd, val, ones, y)
     interior = np.diff(A.pos) == 5
     assert np.all(y.cpu().numpy()[interior] == 0.0)
+
+
+def test_kernel_timing_counts_the_dominant_kernel_launches(gpu):
+    # what bench.py's roofline figure rests on: one event pair per launch of the SpMV main kernel
+    A = gen.laplace2d(64)
+    pos, crd, val = dev(A.pos), dev(A.crd), dev(A.val)
+    x, y = dev(gen.uniform_vector(A.ncols, 3)), dev(np.zeros(A.nrows))
+    plan = gpu.CsrPlan(A.nrows, A.ncols, pos, crd, value_bytes=8)
+    gpu.kernel_timing_start(5)
+    for _ in range(7):  # more launches than capacity: the later ones are not timed
+        gpu.spmv(plan, A.nrows, A.ncols, pos, crd, val, x, y)
+    t = gpu.kernel_timing_stop()
+    assert t["count"] == 5
+    assert 0.0 < t["min_ms"] <= t["median_ms"] <= t["max_ms"] < 50.0
+    assert t["min_ms"] <= t["mean_ms"] <= t["max_ms"]
+    with pytest.raises(gpu.LapisHipError):
+        gpu.kernel_timing_stop()  # not started
