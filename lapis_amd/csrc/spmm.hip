@@ -5,6 +5,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
+#include <type_traits>
 
 #include "common.hpp"
 #include "plan.hpp"
@@ -31,7 +32,7 @@ struct RowVec<double> {
 // handed to the lane groups by bpermute.  The G partial rows are added up with xor
 // shuffles.  VEC = false is the same kernel with element-wise guarded accesses, for k
 // that is no multiple of the vector width and for buffers that are not 16-byte aligned.
-template <typename T, int LPR, bool VEC>
+template <typename T, int LPR, bool VEC, bool DEEP>
 __global__ __launch_bounds__(256) void spmm_wave_row_kernel(int nrows, int k, const int *__restrict__ pos,
                                                             const int *__restrict__ crd,
                                                             const T *__restrict__ val, const T *__restrict__ B,
@@ -56,26 +57,66 @@ __global__ __launch_bounds__(256) void spmm_wave_row_kernel(int nrows, int k, co
       c_l = load_stream(crd + base + lane);
       a_l = load_stream(val + base + lane);
     }
-    // every lane runs every round (the bpermutes need their source lanes active);
-    // a group whose non-zero index falls past the row end sits the round out
-#pragma unroll 8
-    for (int t0 = 0; t0 < cnt; t0 += G) {
-      const int t = t0 + g;
-      const int cj = __shfl(c_l, t & 63, 64);
-      const T aj = __shfl(a_l, t & 63, 64);
-      if (t < cnt && col < k) {
-        const T *bp = B + (long long)cj * ldb + col;
-        if (VEC) {
-          const V b = *reinterpret_cast<const V *>(bp);
+    // Every lane runs every step (the bpermutes need their source lanes active).  With DEEP, steps go
+    // together in batches of 8, 4, 2 and 1: the B rows of a batch are loaded first, without any condition
+    // -- a lane group past the row end reads the row of a lane that holds column 0 and value 0, a lane
+    // past the last column of B reads column 0 -- and then added in order, so a lane keeps up to 8
+    // gathered rows in flight.  (Loads inside the `t < cnt` test are not unrolled by the compiler and
+    // are waited for one by one, which is what !DEEP does: better where B comes from HBM anyway.)
+    const int colc = col < k ? col : 0;
+    auto batch = [&](int t0, auto unr) {
+      constexpr int UNR = decltype(unr)::value;
+      T a[UNR];
+      if (VEC) {
+        V b[UNR];
 #pragma unroll
-          for (int e = 0; e < VW; ++e) acc[e] = acc[e] + aj * b[e];
-        } else {
+        for (int u = 0; u < UNR; ++u) {
+          const int t = t0 + u * G + g;
+          const int cj = __shfl(c_l, t & 63, 64);
+          a[u] = __shfl(a_l, t & 63, 64);
+          b[u] = *reinterpret_cast<const V *>(B + (long long)cj * ldb + colc);
+        }
 #pragma unroll
-          for (int e = 0; e < VW; ++e)
-            if (col + e < k) acc[e] = acc[e] + aj * bp[e];
+        for (int u = 0; u < UNR; ++u) {
+          if (t0 + u * G + g < cnt && col < k) {
+#pragma unroll
+            for (int e = 0; e < VW; ++e) acc[e] = acc[e] + a[u] * b[u][e];
+          }
+        }
+      } else {
+        T b[UNR][VW];
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+          const int t = t0 + u * G + g;
+          const int cj = __shfl(c_l, t & 63, 64);
+          a[u] = __shfl(a_l, t & 63, 64);
+          const T *bp = B + (long long)cj * ldb;
+#pragma unroll
+          for (int e = 0; e < VW; ++e) b[u][e] = bp[col + e < k ? col + e : 0];
+        }
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+          if (t0 + u * G + g < cnt) {
+#pragma unroll
+            for (int e = 0; e < VW; ++e)
+              if (col + e < k) acc[e] = acc[e] + a[u] * b[u][e];
+          }
         }
       }
+    };
+    int t0 = 0;
+    if (DEEP) {
+      for (; t0 + 7 * G < cnt; t0 += 8 * G) batch(t0, std::integral_constant<int, 8>());
+      if (t0 + 3 * G < cnt) {
+        batch(t0, std::integral_constant<int, 4>());
+        t0 += 4 * G;
+      }
+      if (t0 + G < cnt) {
+        batch(t0, std::integral_constant<int, 2>());
+        t0 += 2 * G;
+      }
     }
+    for (; t0 < cnt; t0 += G) batch(t0, std::integral_constant<int, 1>());
   }
 #pragma unroll
   for (int o = LPR; o < 64; o <<= 1) {
@@ -137,14 +178,37 @@ __global__ __launch_bounds__(256) void spmm_group_row_kernel(int nrows, const in
         c_l = load_stream(crd + base + l);
         a_l = load_stream(val + base + l);
       }
-#pragma unroll 8
-      for (int t = 0; t < cnt; ++t) {
-        const int cj = __shfl(c_l, g * LPR + t, 64);  // from a lane of this group: it runs the same trip
-        const T aj = __shfl(a_l, g * LPR + t, 64);
-        const V b = *reinterpret_cast<const V *>(B + (long long)cj * ldb + l * VW);
+      // Non-zeros go together in batches of 8, 4, 2 and 1: the B rows of a batch are loaded first, then
+      // added in order, so a lane keeps up to 8 gathered rows in flight (a loop that loads and adds one
+      // non-zero per trip is not unrolled by the compiler and waits for every row before it asks for the next)
+      auto batch = [&](int t0, auto unr) {
+        constexpr int UNR = decltype(unr)::value;
+        T a[UNR];
+        V b[UNR];
 #pragma unroll
-        for (int e = 0; e < VW; ++e) acc[e] = acc[e] + aj * b[e];
+        for (int u = 0; u < UNR; ++u) {
+          const int src = g * LPR + t0 + u;  // a lane of this group: it runs the same trip
+          const int cj = __shfl(c_l, src, 64);
+          a[u] = __shfl(a_l, src, 64);
+          b[u] = *reinterpret_cast<const V *>(B + (long long)cj * ldb + l * VW);
+        }
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+#pragma unroll
+          for (int e = 0; e < VW; ++e) acc[e] = acc[e] + a[u] * b[u][e];
+        }
+      };
+      int t0 = 0;
+      for (; t0 + 8 <= cnt; t0 += 8) batch(t0, std::integral_constant<int, 8>());
+      if (t0 + 4 <= cnt) {
+        batch(t0, std::integral_constant<int, 4>());
+        t0 += 4;
       }
+      if (t0 + 2 <= cnt) {
+        batch(t0, std::integral_constant<int, 2>());
+        t0 += 2;
+      }
+      if (t0 < cnt) batch(t0, std::integral_constant<int, 1>());
     }
     if (row < nrows) {
       V *cp = reinterpret_cast<V *>(C + row * ldc + l * VW);
@@ -200,7 +264,6 @@ __global__ __launch_bounds__(1024) void spmm_rowblock_lds_kernel(int nrows, int 
         c_l = load_stream(crd + base + lane);
         a_l = load_stream(val + base + lane);
       }
-#pragma unroll 8
       for (int t0 = 0; t0 < cnt; t0 += G) {
         const int t = t0 + g;
         const int cj = __shfl(c_l, t & 63, 64);
@@ -257,28 +320,32 @@ __global__ __launch_bounds__(256) void bspmm_csrv_kernel(int n1, int dh, int nh,
 
 template <typename T, int LPR, bool VEC>
 void launch_wave_row(int64_t nrows, int64_t k, const int *pos, const int *crd, const T *val, const T *B, int64_t ldb,
-                     T *C, int64_t ldc, hipStream_t st) {
+                     T *C, int64_t ldc, hipStream_t st, bool deep) {
   constexpr int VW = RowVec<T>::width;
   const dim3 grid((unsigned)ceil_div(nrows, 4), (unsigned)ceil_div(k, LPR * VW));
-  launch_timed(spmm_wave_row_kernel<T, LPR, VEC>, grid, dim3(256), st, (int)nrows, (int)k, pos, crd, val, B,
-               (long long)ldb, C, (long long)ldc);
+  if (deep)
+    launch_timed(spmm_wave_row_kernel<T, LPR, VEC, true>, grid, dim3(256), st, (int)nrows, (int)k, pos, crd, val, B,
+                 (long long)ldb, C, (long long)ldc);
+  else
+    launch_timed(spmm_wave_row_kernel<T, LPR, VEC, false>, grid, dim3(256), st, (int)nrows, (int)k, pos, crd, val, B,
+                 (long long)ldb, C, (long long)ldc);
 }
 
 template <typename T, bool VEC>
 void launch_wave_row_any(int64_t nrows, int64_t k, const int *pos, const int *crd, const T *val, const T *B, int64_t ldb,
-                         T *C, int64_t ldc, hipStream_t st) {
+                         T *C, int64_t ldc, hipStream_t st, bool deep) {
   constexpr int VW = RowVec<T>::width;
   // lanes per chunk of a B row: the smallest power of two that covers k, at most a wavefront
   int lpr = 1;
   while (lpr < 64 && (int64_t)lpr * VW < k) lpr *= 2;
   switch (lpr) {
-    case 1: launch_wave_row<T, 1, VEC>(nrows, k, pos, crd, val, B, ldb, C, ldc, st); break;
-    case 2: launch_wave_row<T, 2, VEC>(nrows, k, pos, crd, val, B, ldb, C, ldc, st); break;
-    case 4: launch_wave_row<T, 4, VEC>(nrows, k, pos, crd, val, B, ldb, C, ldc, st); break;
-    case 8: launch_wave_row<T, 8, VEC>(nrows, k, pos, crd, val, B, ldb, C, ldc, st); break;
-    case 16: launch_wave_row<T, 16, VEC>(nrows, k, pos, crd, val, B, ldb, C, ldc, st); break;
-    case 32: launch_wave_row<T, 32, VEC>(nrows, k, pos, crd, val, B, ldb, C, ldc, st); break;
-    default: launch_wave_row<T, 64, VEC>(nrows, k, pos, crd, val, B, ldb, C, ldc, st); break;
+    case 1: launch_wave_row<T, 1, VEC>(nrows, k, pos, crd, val, B, ldb, C, ldc, st, deep); break;
+    case 2: launch_wave_row<T, 2, VEC>(nrows, k, pos, crd, val, B, ldb, C, ldc, st, deep); break;
+    case 4: launch_wave_row<T, 4, VEC>(nrows, k, pos, crd, val, B, ldb, C, ldc, st, deep); break;
+    case 8: launch_wave_row<T, 8, VEC>(nrows, k, pos, crd, val, B, ldb, C, ldc, st, deep); break;
+    case 16: launch_wave_row<T, 16, VEC>(nrows, k, pos, crd, val, B, ldb, C, ldc, st, deep); break;
+    case 32: launch_wave_row<T, 32, VEC>(nrows, k, pos, crd, val, B, ldb, C, ldc, st, deep); break;
+    default: launch_wave_row<T, 64, VEC>(nrows, k, pos, crd, val, B, ldb, C, ldc, st, deep); break;
   }
 }
 
@@ -411,10 +478,16 @@ int spmm_impl(const char *what, const lapis_hip_csr_plan *plan, int64_t nrows, i
     }
   }
   g_last_spmm_kernel = "spmm_wave_row_kernel";
+  // Several gathered B rows in flight per lane pay where B rows come from L2 (columns of a chunk of A within
+  // 32 MB of B, or no plan to say otherwise); where every gather goes to HBM they only get in each other's way
+  // (config 4 of the benchmarks: 1.21 ms one at a time, 1.26 ms eight at a time).
+  bool deep = true;
+  if (plan) deep = plan->stats.mean_chunk_col_span * (double)k * sizeof(T) <= 32.0 * 1024 * 1024;
+  if (const char *d = getenv("LAPIS_HIP_SPMM_DEEP")) deep = atoi(d) != 0;
   if (vec)
-    launch_wave_row_any<T, true>(nrows, k, pos, crd, val, B, ldb, C, ldc, st);
+    launch_wave_row_any<T, true>(nrows, k, pos, crd, val, B, ldb, C, ldc, st, deep);
   else
-    launch_wave_row_any<T, false>(nrows, k, pos, crd, val, B, ldb, C, ldc, st);
+    launch_wave_row_any<T, false>(nrows, k, pos, crd, val, B, ldb, C, ldc, st, deep);
   LAPIS_LAUNCH_CHECK();
   return LAPIS_HIP_OK;
 }
