@@ -169,11 +169,12 @@ void laplace3d(int n, Csr &A) {
 
 int main(int argc, const char **argv) {
   std::vector<std::string> positional;
-  bool check = false;
+  bool check = false, parse_only = false;
   std::string dump_path;
   for (int i = 1; i < argc; ++i) {
     const std::string a = argv[i];
     if (a == "--check") check = true;
+    else if (a == "--parse-only") parse_only = true;
     else if (a == "--dump-y" && i + 1 < argc) dump_path = argv[++i];
     else if (a.rfind("--", 0) == 0) {
       std::cerr << "unknown option " << a << "\n";
@@ -181,13 +182,12 @@ int main(int argc, const char **argv) {
     } else positional.push_back(a);
   }
   if (positional.empty() || positional.size() > 3) {
-    std::cout << "Expected: matrix file in MatrixMarket format [trials] [kernel] [--check] [--dump-y FILE]\n";
+    std::cout << "Expected: matrix file in MatrixMarket format [trials] [kernel] [--check] [--dump-y FILE] [--parse-only]\n";
     return 1;
   }
   const std::string mfile = positional[0];
   const int trials = positional.size() > 1 ? std::max(1, atoi(positional[1].c_str())) : 1000;
   const std::string kernel = positional.size() > 2 ? positional[2] : "auto";
-  CHECK_LAPIS(lapis_hip_init());
   Csr A;
   std::string err;
   if (mfile.rfind("gen:laplace3d:", 0) == 0) {
@@ -207,6 +207,24 @@ int main(int argc, const char **argv) {
   }
   const int64_t nnz = (int64_t)A.crd.size();
   std::cout << "Read matrix (" << A.nrows << "x" << A.ncols << " with " << nnz << " entries)\n";
+  if (parse_only) {
+    // what the reader made of the file, without touching the GPU: sums that change with a dropped, doubled,
+    // transposed or sign-flipped entry, and whether every row's columns ascend
+    double sum = 0.0, weighted = 0.0;
+    bool sorted = true;
+    for (int64_t r = 0; r < A.nrows; ++r)
+      for (int64_t j = A.pos[r]; j < A.pos[r + 1]; ++j) {
+        sum += A.val[j];
+        weighted += (double)(r + 1) * (double)(2 * (int64_t)A.crd[j] + 1) * A.val[j];
+        if (j > A.pos[r] && A.crd[j] <= A.crd[j - 1]) sorted = false;
+      }
+    std::cout.precision(17);
+    std::cout << "parse: sum(val) = " << sum << "\n";
+    std::cout << "parse: sum((row+1)*(2*col+1)*val) = " << weighted << "\n";
+    std::cout << "parse: columns ascend in every row = " << (sorted ? "yes" : "no") << "\n";
+    return 0;
+  }
+  CHECK_LAPIS(lapis_hip_init());
 
   int32_t *pos = nullptr, *crd = nullptr;
   double *val = nullptr, *x = nullptr, *y = nullptr;
