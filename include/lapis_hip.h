@@ -242,7 +242,7 @@ int lapis_hip_spmm_csr_f64_i32(int64_t nrows, int64_t ncols, int64_t k, const in
  *   group per row: matrices with short, even rows (mean <= 256, longest <= 4 x mean)
  *     whose columns stay local (the B rows a stretch of 1024 non-zeros touches fit the
  *     L2s: stencils, meshes).  64/LPR rows per wavefront at a time, one group of lanes
- *     per row, no cross-lane reduction: 1.2x-4.5x faster than the kernel below there.
+ *     per row, no cross-lane reduction: 1.25x-5.8x faster than the kernel below there.
  *   wavefront per row: everything else, and `plan == NULL` (the entry points above).
  *   LDS-staged row block: a workgroup stages the rows of B of its block's diagonal
  *     window in LDS with coalesced 128-bit loads and serves the non-zeros inside the

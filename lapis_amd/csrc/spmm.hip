@@ -126,10 +126,10 @@ __global__ __launch_bounds__(256) void spmm_wave_row_kernel(int nrows, int k, co
   if (g == 0 && col < k) {
     T *cp = C + row * ldc + col;
     if (VEC) {
-      V cin = *reinterpret_cast<V *>(cp);
+      V cin = load_stream(reinterpret_cast<V *>(cp));
 #pragma unroll
       for (int e = 0; e < VW; ++e) cin[e] = acc[e] + cin[e];
-      *reinterpret_cast<V *>(cp) = cin;
+      store_stream(reinterpret_cast<V *>(cp), cin);
     } else {
 #pragma unroll
       for (int e = 0; e < VW; ++e)
@@ -139,7 +139,7 @@ __global__ __launch_bounds__(256) void spmm_wave_row_kernel(int nrows, int k, co
 }
 
 // One group of LPR lanes per row of A: a wavefront works on G = 64/LPR rows at a time,
-// ROUNDS times over.  Each group walks its own row, LPR non-zeros per coalesced read of
+// ROUNDS times over (once by default).  Each group walks its own row, LPR non-zeros per coalesced read of
 // crd/val, one B row (LPR 128-bit loads) per non-zero, and keeps the row of C in its own
 // registers: no reduction across lanes, G rows of loads in flight per instruction, and
 // the G rows of C a wavefront writes are neighbours.  For short, even rows (stencils,
@@ -212,10 +212,10 @@ __global__ __launch_bounds__(256) void spmm_group_row_kernel(int nrows, const in
     }
     if (row < nrows) {
       V *cp = reinterpret_cast<V *>(C + row * ldc + l * VW);
-      V cin = *cp;
+      V cin = load_stream(cp);
 #pragma unroll
       for (int e = 0; e < VW; ++e) cin[e] = acc[e] + cin[e];
-      *cp = cin;
+      store_stream(cp, cin);
     }
   }
 }
@@ -349,10 +349,9 @@ void launch_wave_row_any(int64_t nrows, int64_t k, const int *pos, const int *cr
   }
 }
 
-template <typename T, int LPR>
-void launch_group_row(int64_t nrows, const int *pos, const int *crd, const T *val, const T *B, int64_t ldb, T *C,
-                      int64_t ldc, hipStream_t st) {
-  constexpr int ROUNDS = 4;
+template <typename T, int LPR, int ROUNDS>
+void launch_group_row_r(int64_t nrows, const int *pos, const int *crd, const T *val, const T *B, int64_t ldb, T *C,
+                        int64_t ldc, hipStream_t st) {
   constexpr int rows_per_block = 4 * (64 / LPR) * ROUNDS;
   const char *xcd = getenv("LAPIS_HIP_SPMM_XCD_MAP");
   if (xcd && atoi(xcd) == 0)
@@ -361,6 +360,18 @@ void launch_group_row(int64_t nrows, const int *pos, const int *crd, const T *va
   else
     launch_timed(spmm_group_row_kernel<T, LPR, ROUNDS, true>, dim3((unsigned)ceil_div(nrows, rows_per_block)), dim3(256),
                  st, (int)nrows, pos, crd, val, B, (long long)ldb, C, (long long)ldc);
+}
+
+template <typename T, int LPR>
+void launch_group_row(int64_t nrows, const int *pos, const int *crd, const T *val, const T *B, int64_t ldb, T *C,
+                      int64_t ldc, hipStream_t st) {
+  // Rounds of rows per wavefront.  One is fastest now that a lane keeps several B rows in flight (Laplace3D_100
+  // k = 64: 0.195 / 0.196 / 0.209 ms with 1 / 2 / 4 rounds; Elasticity3D_60: 0.606 / 0.623 / 0.649 ms): the fewer
+  // rows an XCD has in flight, the smaller the part of B its L2 has to hold.  LAPIS_HIP_SPMM_ROUNDS = 2, 4 for tuning.
+  const int rounds = getenv("LAPIS_HIP_SPMM_ROUNDS") ? atoi(getenv("LAPIS_HIP_SPMM_ROUNDS")) : 1;
+  if (rounds == 4) launch_group_row_r<T, LPR, 4>(nrows, pos, crd, val, B, ldb, C, ldc, st);
+  else if (rounds == 2) launch_group_row_r<T, LPR, 2>(nrows, pos, crd, val, B, ldb, C, ldc, st);
+  else launch_group_row_r<T, LPR, 1>(nrows, pos, crd, val, B, ldb, C, ldc, st);
 }
 
 constexpr int kSpmmLdsBytes = 128 * 1024;  // staged rows of B per workgroup of the LDS kernel
