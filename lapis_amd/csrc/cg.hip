@@ -247,7 +247,9 @@ __global__ __launch_bounds__(256) void cg_precond_kernel(long long n, const doub
   double acc = 0.0;
   const long long nv = vec ? n / 2 : 0;
   CG_GRID_STRIDE(i, 0, nv) {
-    const v2d rv = ld2(r, i), dv = ld2(dinv, i);
+    // r and the preconditioner are read here for the last time in this iteration
+    const v2d rv = load_stream(reinterpret_cast<const v2d *>(r) + i);
+    const v2d dv = load_stream(reinterpret_cast<const v2d *>(dinv) + i);
     v2d zv;
     zv.x = divide ? rv.x / dv.x : rv.x * dv.x;
     zv.y = divide ? rv.y / dv.y : rv.y * dv.y;
