@@ -56,7 +56,9 @@ def calibrate_gather(full=False):
     import torch
     from lapis_amd import hip
     gathers = 1 << 26
-    stream = torch.zeros(1 << 27, dtype=torch.float64, device="cuda")  # 1 GiB: 12 bytes per gather fit
+    # 1 GiB: 12 bytes per gather fit; the full table has modes in which only half of the wavefronts stream,
+    # each from a region of its own
+    stream = torch.zeros(1 << (28 if full else 27), dtype=torch.float64, device="cuda")
     x = torch.zeros(1 << 23, dtype=torch.float64, device="cuda")       # 64 MB window at most
     sink = torch.zeros(4096, dtype=torch.float64, device="cuda")
     l2 = 1 << 20
@@ -84,7 +86,55 @@ def calibrate_gather(full=False):
                                   "predicted_ms": (r["stream_bytes"] / stream_rate + lines / line_rate) * 1e3
                                   if window == l2 else None})
         out["table"] = table
+        out["modes"] = calibrate_modes(hip, x, l2, stream, sink, stream_rate, line_rate)
     del stream, x, sink
+    return out
+
+
+def calibrate_modes(hip, x, window, stream, sink, stream_rate, line_rate):
+    """The same stream and the same gathers in other arrangements (lapis_hip_calibrate_mix): does any of them let
+    a compute unit overlap the two?  805 MB of stream and 42.4 M single-line gathers from an L2-resident window --
+    what config 2 sends after the column-blocked copy has merged its gathers -- unless a row says otherwise."""
+    import torch
+    cu_count = torch.zeros(16 * 256, dtype=torch.int32, device="cuda")
+    S, G = 12 << 26, 42.4e6
+    both = lambda **kw: dict(kw)
+    rows = [
+        ("stream only", both(threads=512, stream_in_flight=3, stream_policy=1), S, 0),
+        ("stream only, 16 wavefronts, 12 loads in flight", both(threads=1024, stream_in_flight=12, stream_policy=1), S, 0),
+        ("stream only, on 64 compute units", both(threads=1024, workgroups=64, stream_in_flight=12, stream_policy=1), S, 0),
+        ("gathers only", both(threads=512, gathers_in_flight=4), 0, G),
+        ("gathers only, 16 wavefronts, 8 in flight", both(threads=1024, gathers_in_flight=8), 0, G),
+        ("every wavefront does both, 8 per CU", both(threads=512, stream_in_flight=3, gathers_in_flight=2, stream_policy=1), S, G),
+        ("every wavefront does both, 16 per CU", both(threads=1024, stream_in_flight=6, gathers_in_flight=4, stream_policy=1), S, G),
+        ("every wavefront does both, 2 workgroups of 8 per CU", both(threads=512, workgroups=512, stream_in_flight=6, gathers_in_flight=4, stream_policy=1), S, G),
+        ("both, next step's stream issued behind the gathers", both(threads=1024, stream_in_flight=6, gathers_in_flight=4, stream_policy=1, stream_behind=1), S, G),
+        ("roles by wavefront: 4 stream, 12 gather", both(threads=1024, stream_in_flight=6, gathers_in_flight=4, stream_policy=1, roles=1, producers=4), S, G),
+        ("roles by wavefront: 4 stream (12 in flight), 8 gather", both(threads=768, stream_in_flight=12, gathers_in_flight=4, stream_policy=1, roles=1, producers=4), S, G),
+        ("roles by wavefront: 8 stream, 8 gather", both(threads=1024, stream_in_flight=6, gathers_in_flight=4, stream_policy=1, roles=1, producers=8), S, G),
+        ("roles by wavefront: 3 stream, 5 gather", both(threads=512, stream_in_flight=12, gathers_in_flight=4, stream_policy=1, roles=1, producers=3), S, G),
+        ("roles by workgroup: 2 x 8 wavefronts per CU", both(threads=512, workgroups=512, stream_in_flight=6, gathers_in_flight=4, stream_policy=1, roles=2), S, G),
+        ("roles by workgroup: 2 x 4 wavefronts per CU", both(threads=256, workgroups=512, stream_in_flight=12, gathers_in_flight=4, stream_policy=1, roles=2), S, G),
+        ("both, stream loads sc0 sc1", both(threads=1024, stream_in_flight=6, gathers_in_flight=4, stream_policy=2), S, G),
+        ("both, stream loads sc0 sc1 nt", both(threads=1024, stream_in_flight=6, gathers_in_flight=4, stream_policy=3), S, G),
+        ("both, stream straight to LDS", both(threads=1024, stream_in_flight=6, gathers_in_flight=4, stream_policy=4), S, G),
+        ("roles by wavefront, stream straight to LDS", both(threads=768, stream_in_flight=12, gathers_in_flight=4, stream_policy=4, roles=1, producers=4), S, G),
+        ("stream kept in L2, alone", both(threads=512, stream_in_flight=3, stream_in_l2=1), S, 0),
+        ("stream kept in L2 + gathers (a perfect prefetch)", both(threads=512, stream_in_flight=3, gathers_in_flight=2, stream_in_l2=1), S, G),
+        ("stream alone through the scalar cache (64-byte loads)", both(threads=1024, workgroups=512, stream_in_flight=3, scalar=1), S // 4, 0),
+        ("both + helper wavefronts touching the stream through the scalar cache, every 128 B", both(threads=512, stream_in_flight=3, gathers_in_flight=4, scalar=2, scalar_ahead=4, scalar_stride=128), S, G),
+        ("both + helper wavefronts touching the stream through the scalar cache, every 64 B", both(threads=512, stream_in_flight=3, gathers_in_flight=4, scalar=2, scalar_ahead=4, scalar_stride=64), S, G),
+        ("stream + such helpers, no gathers", both(threads=512, stream_in_flight=3, scalar=2, scalar_ahead=4, scalar_stride=128), S, 0),
+    ]
+    out = []
+    for label, mode, sbytes, gathers in rows:
+        r = hip.calibrate_mix(mode, x, window, stream, sbytes, gathers, cu_count, sink)
+        lines = r["gathers"]
+        out.append({"mode": label, "ms": r["ms"], "stream_MB": r["stream_bytes"] / 1e6, "gather_lines_M": lines / 1e6,
+                    "stream_TB_per_s": r["stream_bytes"] / (r["ms"] * 1e-3) / 1e12,
+                    "gather_lines_G_per_s": lines / (r["ms"] * 1e-3) / 1e9,
+                    "sum_of_parts_ms": (r["stream_bytes"] / stream_rate + lines / line_rate) * 1e3,
+                    "cus_with_both_roles": r["cus_with_both_roles"], **mode})
     return out
 
 

@@ -80,6 +80,37 @@ int lapis_hip_calibrate_gather(const double *x, int64_t window_bytes, int lanes_
                                int64_t stream_bytes, int64_t gathers, double *sink, double *elapsed_ms,
                                double *gathers_done, double *stream_bytes_done, lapis_hip_stream_t stream);
 
+/* Measurement only (`bench.py --calibrate-gather`): the same two kinds of load in other
+ * arrangements, to see whether any of them lets a compute unit overlap the stream with the
+ * gathers.  A launch streams `stream_bytes` from `stream_buf` and does `gathers` gathers of
+ * doubles from the first `window_bytes` of `x`, split evenly over the wavefronts that have
+ * the role.  `cu_count` (16 * 256 ints) is needed for roles = 2 only.  Returns the best of
+ * five timed launches and what one launch did; `cus_with_both_roles` = compute units that
+ * ran one workgroup of each role (roles = 2), else -1.  No counterpart in the reference. */
+typedef struct lapis_hip_calibrate_mode {
+  int threads;           /* per workgroup, a multiple of 64 up to 1024 */
+  int workgroups;        /* 0 = one per compute unit */
+  int stream_in_flight;  /* 16-byte loads per lane and step: 0 (no stream), 3, 6 or 12 */
+  int gathers_in_flight; /* gathers per lane and step: 0 (none), 2, 4 or 8 */
+  int lanes_per_line;    /* neighbouring lanes of a gather instruction in one 128-byte line */
+  int roles;             /* 0: every wavefront streams and gathers; 1: `producers` wavefronts of each
+                            workgroup only stream, the others only gather; 2: by workgroup, in the
+                            order in which workgroups arrive on a compute unit */
+  int producers;
+  int stream_behind;     /* 1: the stream loads of the next step are issued after this step's gathers */
+  int stream_policy;     /* 0 plain, 1 nt, 2 sc0 sc1, 3 sc0 sc1 nt, 4 straight to LDS */
+  int stream_in_l2;      /* 1: the stream wraps inside a window that stays in L2 */
+  int scalar;            /* 1: the stream alone, read with 64-byte scalar loads; 2: as many helper
+                            wavefronts as consumers touch the consumers' stream through the scalar
+                            cache `scalar_ahead` steps ahead, one 4-byte load per `scalar_stride` bytes */
+  int scalar_ahead;
+  int scalar_stride;
+} lapis_hip_calibrate_mode;
+int lapis_hip_calibrate_mix(const lapis_hip_calibrate_mode *mode, const double *x, int64_t window_bytes,
+                            const void *stream_buf, int64_t stream_buf_bytes, int64_t stream_bytes, int64_t gathers,
+                            int *cu_count, double *sink, double *elapsed_ms, double *gathers_done,
+                            double *stream_bytes_done, int *cus_with_both_roles, lapis_hip_stream_t stream);
+
 /* ---- CSR plan: the team/vector loop-mapping decision ---------------------- */
 
 /* Which kernel a plan launches for SpMV. */
@@ -160,6 +191,13 @@ int lapis_hip_csr_plan_analyze(lapis_hip_csr_plan *plan, const int32_t *crd, con
  * alone (status OK). */
 int lapis_hip_csr_plan_update_values(lapis_hip_csr_plan *plan, const void *val, int value_bytes,
                                      lapis_hip_stream_t stream);
+/* Waits for `stream` and reports whether a kernel of this plan gave up a wait between its
+ * own wavefronts (the workgroup-blocked SpMV hands entries from streaming wavefronts to
+ * gathering ones through LDS, and every such wait is bounded so that a launch always
+ * ends): LAPIS_HIP_OK, or LAPIS_HIP_ERR_RUNTIME, in which case the last results computed
+ * with the plan are not to be used.  No counterpart in the reference; for tests and for
+ * callers that want the assurance. */
+int lapis_hip_csr_plan_check(lapis_hip_csr_plan *plan, lapis_hip_stream_t stream);
 /* Overrides the automatic choice (tuning and tests).  `width` is used by SUBWARP
  * (0 = the reference's rule); other kernels ignore it. */
 int lapis_hip_csr_plan_set_kernel(lapis_hip_csr_plan *plan, int kernel, int width);

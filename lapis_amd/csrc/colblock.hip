@@ -264,6 +264,9 @@ void free_colblock(lapis_hip_csr_plan *p) {
   if (p->colblock_tile_ptr) (void)hipFree(p->colblock_tile_ptr);
   if (p->colblock_units) (void)hipFree(p->colblock_units);
   if (p->colblock_long_rows) (void)hipFree(p->colblock_long_rows);
+  if (p->colblock_fault) (void)hipFree(p->colblock_fault);
+  p->colblock_fault = nullptr;
+  p->colblock_pc_prod = 0;
   p->colblock_tile_ptr = nullptr;
   p->colblock_units = nullptr;
   p->colblock_long_rows = nullptr;
@@ -531,6 +534,20 @@ extern "C" int lapis_hip_csr_plan_update_values(lapis_hip_csr_plan *plan, const 
                                             static_cast<float *>(plan->colblock_val), plan->stats.nnz, st);
   if (rc == LAPIS_HIP_OK) plan->colblock_src_val = val;
   return rc;
+}
+
+extern "C" int lapis_hip_csr_plan_check(lapis_hip_csr_plan *plan, lapis_hip_stream_t stream) {
+  LAPIS_CHECK_INIT();
+  LAPIS_REQUIRE(plan, "csr_plan_check: null plan");
+  hipStream_t st = as_stream(stream);
+  LAPIS_HIP_TRY(hipStreamSynchronize(st));
+  if (!plan->colblock_fault) return LAPIS_HIP_OK;
+  int fault = 0;
+  LAPIS_HIP_TRY(hipMemcpy(&fault, plan->colblock_fault, sizeof(int), hipMemcpyDeviceToHost));
+  if (fault != 0)
+    return set_error(LAPIS_HIP_ERR_RUNTIME,
+                     "csr_plan_check: a wavefront of the workgroup-blocked SpMV gave up waiting for its partner");
+  return LAPIS_HIP_OK;
 }
 
 extern "C" int lapis_hip_csr_plan_analyze(lapis_hip_csr_plan *plan, const int32_t *crd, const void *val, int value_bytes,

@@ -154,6 +154,205 @@ __global__ __launch_bounds__(THREADS) void spmv_colgroup_kernel(int nrows, int r
   }
 }
 
+// ---- the same walk with producer and consumer wavefronts -------------------------------
+//
+// A wavefront that both streams its entries and gathers x waits, at every step, for
+// whatever it has in flight: loads of one wavefront return in issue order, so the wait
+// for a gather that hits L2 is also a wait for the entry loads issued before it, which
+// come from HBM.  Here the roles are split.  PROD wavefronts of the workgroup only
+// stream: 512 entries (index words and values, 128-bit loads) per step, two steps in
+// flight, handed over through a ring of kPcSlots x 512 entries in LDS.  The other
+// wavefronts only consume: they copy a chunk from the ring into registers, give the slot
+// back, gather x and add into the row sums.  Chunk k is loaded by producer k % PROD,
+// passes through slot k % kPcSlots and is consumed by consumer k % CONS; `ready[slot]`
+// and `taken[slot]` count how often the slot was filled and emptied.  LDS operations of a
+// wavefront execute in issue order, so a flag written after the data is seen after it.
+// Every wait is bounded: a flag that never comes makes the wavefront give up and set
+// *fault (lapis_hip_csr_plan_check reports it), so the grid drains whatever happens.
+constexpr int kPcChunk = 512;
+constexpr int kPcSlots = 4;
+constexpr int kPcPad = 1024;  // entries allocated behind the copy: the last chunk is loaded whole
+
+// The flags are read and written with the LDS instructions themselves: a volatile access would make the
+// compiler wait for every load the wavefront has in flight, the producers' next chunk included.
+typedef __attribute__((address_space(3))) int lds_int;
+__device__ __forceinline__ int pc_flag_load(const int *flag) {
+  int v;
+  const unsigned a = (unsigned)(uintptr_t)(const lds_int *)flag;
+  asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(a) : "memory");
+  return v;
+}
+__device__ __forceinline__ void pc_flag_store(int *flag, int v) {
+  const unsigned a = (unsigned)(uintptr_t)(lds_int *)flag;
+  asm volatile("ds_write_b32 %0, %1" : : "v"(a), "v"(v) : "memory");
+}
+
+__device__ __forceinline__ bool pc_wait(const int *flag, int want) {
+  for (int spin = 0; spin < (1 << 22); ++spin) {
+    const int v = __builtin_amdgcn_readfirstlane(pc_flag_load(flag));
+    if (v == want) return true;
+    __builtin_amdgcn_s_sleep(1);
+  }
+  return false;
+}
+
+__device__ __forceinline__ void pc_compiler_fence() { __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront"); }
+
+template <typename T> struct PcVal;
+template <> struct PcVal<double> { typedef v2d vec; static constexpr int per = 2; };
+template <> struct PcVal<float> { typedef v4f vec; static constexpr int per = 4; };
+
+template <typename T, int THREADS, int PROD, bool NT>
+__global__ __launch_bounds__(THREADS) void spmv_colgroup_pc_kernel(int nrows, int rows_per_block, int nblocks_nat,
+                                                                   int nlong, int nslices, int slice_log2,
+                                                                   const int *__restrict__ units,
+                                                                   const int *__restrict__ tile_ptr,
+                                                                   const int *__restrict__ long_rows,
+                                                                   const unsigned *__restrict__ bidx,
+                                                                   const T *__restrict__ bval, const T *__restrict__ x,
+                                                                   T *__restrict__ y, int *__restrict__ fault) {
+  typedef typename PcVal<T>::vec VV;
+  constexpr int VPER = PcVal<T>::per;            // values per 16-byte vector
+  constexpr int NIV = kPcChunk / (64 * 4);       // index vectors per lane and chunk (2)
+  constexpr int NVV = kPcChunk / (64 * VPER);    // value vectors per lane and chunk (4 fp64, 2 fp32)
+  constexpr int EPL = kPcChunk / 64;             // entries per consumer lane and chunk (8)
+  constexpr int CONS = THREADS / 64 - PROD;
+  constexpr int DEPTH = 2;                       // chunks a producer has in flight (4 measured slower)
+  static_assert(CONS >= 1 && PROD >= 1, "both roles need a wavefront");
+  extern __shared__ __align__(16) unsigned char colgroup_lds[];
+  double *acc = reinterpret_cast<double *>(colgroup_lds);
+  T *rval = reinterpret_cast<T *>(acc + rows_per_block);
+  unsigned *ridx = reinterpret_cast<unsigned *>(rval + kPcSlots * kPcChunk);
+  int *ready = reinterpret_cast<int *>(ridx + kPcSlots * kPcChunk);
+  int *taken = ready + kPcSlots;
+  int *tp = taken + kPcSlots;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int block = units[4 * blockIdx.x];
+  const int e_first = units[4 * blockIdx.x + 1];
+  const int e_last = units[4 * blockIdx.x + 2];
+  const int sole = units[4 * blockIdx.x + 3];
+  for (int i = tid; i < rows_per_block; i += THREADS) acc[i] = 0.0;
+  {
+    const int *gtp = tile_ptr + (long long)block * (nslices + 1);
+    for (int i = tid; i <= nslices; i += THREADS) tp[i] = gtp[i];
+  }
+  if (tid < 2 * kPcSlots) ready[tid] = 0;  // ready[] and taken[] are neighbours
+  __syncthreads();
+
+  const int base0 = e_first & ~3;  // chunks start on 16-byte boundaries of both arrays
+  const int nchunks = e_last > e_first ? (e_last - base0 + kPcChunk - 1) / kPcChunk : 0;
+  bool ok = true;
+  if (wave < PROD) {
+    v4i ci[DEPTH][NIV];
+    VV cv[DEPTH][NVV];
+    auto load_chunk = [&](int k, v4i (&li)[NIV], VV (&lv)[NVV]) {
+      const long long cb = (long long)base0 + (long long)k * kPcChunk;
+      const v4i *pi = reinterpret_cast<const v4i *>(bidx + cb) + lane;
+      const VV *pv = reinterpret_cast<const VV *>(bval + cb) + lane;
+#pragma unroll
+      for (int j = 0; j < NIV; ++j) li[j] = ldv<NT>(pi + j * 64);
+#pragma unroll
+      for (int j = 0; j < NVV; ++j) lv[j] = ldv<NT>(pv + j * 64);
+    };
+    // chunk k: wait until its slot was emptied, copy it there, say so
+    auto hand_over = [&](int k, const v4i (&li)[NIV], const VV (&lv)[NVV]) {
+      const int slot = k % kPcSlots, round = k / kPcSlots;
+      if (!pc_wait(taken + slot, round)) return false;
+      pc_compiler_fence();
+      v4i *wi = reinterpret_cast<v4i *>(ridx + slot * kPcChunk) + lane;
+      VV *wv = reinterpret_cast<VV *>(rval + slot * kPcChunk) + lane;
+#pragma unroll
+      for (int j = 0; j < NIV; ++j) wi[j * 64] = li[j];
+#pragma unroll
+      for (int j = 0; j < NVV; ++j) wv[j * 64] = lv[j];
+      pc_compiler_fence();
+      pc_flag_store(ready + slot, round + 1);
+      return true;
+    };
+    // two register sets taken in turns, so that the loads of one chunk stay in flight while the
+    // other goes to the ring (a copy from one set to the other would wait for them)
+    // DEPTH register sets taken in turns: the loads of the others stay in flight while one goes to the
+    // ring (a copy between sets would wait for them).  The refill is unconditional (past the end it
+    // repeats the last chunk, which nobody takes): behind a condition the compiler no longer knows how
+    // many loads are in flight and waits for all of them.
+    if (wave < nchunks) {
+      int k = wave;
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) load_chunk(min(k + d * PROD, nchunks - 1), ci[d], cv[d]);
+      while (ok && k < nchunks) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+          if (ok && k < nchunks) ok = hand_over(k, ci[d], cv[d]);
+          load_chunk(min(k + DEPTH * PROD, nchunks - 1), ci[d], cv[d]);
+          k += PROD;
+        }
+      }
+    }
+  } else {
+    const int c = wave - PROD;
+    const unsigned cmask = (1u << slice_log2) - 1u;
+    // the slice of this lane's entries: tp[s] <= position < tp[s + 1]; positions only grow
+    int s = 0, nb = tp[1];
+    for (int k = c; k < nchunks && ok; k += CONS) {
+      const int slot = k % kPcSlots, round = k / kPcSlots;
+      ok = pc_wait(ready + slot, round + 1);
+      if (!ok) break;
+      pc_compiler_fence();
+      unsigned w[EPL];
+      T v[EPL];
+#pragma unroll
+      for (int u = 0; u < EPL; ++u) {
+        w[u] = ridx[slot * kPcChunk + u * 64 + lane];
+        v[u] = rval[slot * kPcChunk + u * 64 + lane];
+      }
+      pc_compiler_fence();
+      pc_flag_store(taken + slot, round + 1);
+      const int cb = base0 + k * kPcChunk;
+      T xv[EPL];
+      bool act[EPL];
+      unsigned xi[EPL];  // an entry outside the unit's range reads x[0] and adds nothing
+#pragma unroll
+      for (int u = 0; u < EPL; ++u) {
+        const int p = cb + u * 64 + lane;
+        act[u] = p >= e_first && p < e_last;
+        xi[u] = 0;
+        if (act[u]) {
+          while (p >= nb) {
+            ++s;
+            nb = tp[s + 1];
+          }
+          xi[u] = ((unsigned)s << slice_log2) + (w[u] & cmask);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < EPL; ++u) xv[u] = x[xi[u]];
+#pragma unroll
+      for (int u = 0; u < EPL; ++u) {
+        const T pr = v[u] * xv[u];
+        if (act[u]) lds_add(acc + (w[u] >> slice_log2), (double)pr);
+      }
+    }
+  }
+  if (!ok && lane == 0) atomicExch(fault, 1);
+  __syncthreads();
+  if (block < nblocks_nat) {
+    const long long row0 = (long long)block * rows_per_block;
+    const int rows_here = (int)std::min<long long>(rows_per_block, nrows - row0);
+    if (sole) {
+      for (int i = tid; i < rows_here; i += THREADS)
+        if (acc[i] != 0.0) y[row0 + i] = T(acc[i]) + y[row0 + i];
+    } else {
+      for (int i = tid; i < rows_here; i += THREADS)
+        if (acc[i] != 0.0) unsafeAtomicAdd(y + row0 + i, T(acc[i]));
+    }
+  } else {
+    const long long base = (long long)(block - nblocks_nat) * rows_per_block;
+    const int rows_here = (int)std::min<long long>(rows_per_block, nlong - base);
+    for (int i = tid; i < rows_here; i += THREADS)
+      if (acc[i] != 0.0) unsafeAtomicAdd(y + long_rows[base + i], T(acc[i]));
+  }
+}
+
 // ---- plan-time kernels ---------------------------------------------------------
 
 __global__ __launch_bounds__(256) void long_row_flag_kernel(int nrows, int long_threshold,
@@ -270,9 +469,66 @@ int launch_colgroup_threads(const lapis_hip_csr_plan *p, const T *x, T *y, hipSt
             : launch_colgroup_cfg<T, THREADS, 8, false>(p, x, y, st);
 }
 
+size_t colgroup_pc_lds_bytes(int rows, int nslices, int value_bytes) {
+  return sizeof(double) * (size_t)rows + (size_t)kPcSlots * kPcChunk * (value_bytes + 4) + sizeof(int) * 2 * kPcSlots +
+         sizeof(int) * ((size_t)nslices + 2);
+}
+
+template <typename T, int THREADS, int PROD, bool NT>
+int launch_colgroup_pc_cfg(const lapis_hip_csr_plan *p, const T *x, T *y, hipStream_t st) {
+  auto kernel = spmv_colgroup_pc_kernel<T, THREADS, PROD, NT>;
+  const size_t lds_bytes = colgroup_pc_lds_bytes(p->colblock_rows, p->colblock_nslices, (int)sizeof(T));
+  static std::once_flag attribute_once;
+  static hipError_t attribute_status = hipSuccess;
+  std::call_once(attribute_once, [&] {
+    attribute_status = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  });
+  LAPIS_HIP_TRY(attribute_status);
+  const dim3 grid((unsigned)p->colblock_nunits), block(THREADS);
+  hipEvent_t e0, e1;
+  if (timing_next_events(&e0, &e1))
+    hipExtLaunchKernelGGL(kernel, grid, block, lds_bytes, st, e0, e1, 0, (int)p->stats.nrows, p->colblock_rows,
+                          p->colblock_nblocks_nat, p->colblock_nlong, p->colblock_nslices, p->colblock_slice_log2,
+                          (const int *)p->colblock_units, (const int *)p->colblock_tile_ptr,
+                          (const int *)p->colblock_long_rows, (const unsigned *)p->colblock_idx,
+                          (const T *)p->colblock_val, x, y, p->colblock_fault);
+  else
+    hipLaunchKernelGGL(kernel, grid, block, lds_bytes, st, (int)p->stats.nrows, p->colblock_rows,
+                       p->colblock_nblocks_nat, p->colblock_nlong, p->colblock_nslices, p->colblock_slice_log2,
+                       (const int *)p->colblock_units, (const int *)p->colblock_tile_ptr,
+                       (const int *)p->colblock_long_rows, (const unsigned *)p->colblock_idx,
+                       (const T *)p->colblock_val, x, y, p->colblock_fault);
+  LAPIS_LAUNCH_CHECK();
+  return LAPIS_HIP_OK;
+}
+
+template <typename T>
+int launch_colgroup_pc(const lapis_hip_csr_plan *p, const T *x, T *y, hipStream_t st) {
+  const bool nt = p->nontemporal;
+#define LAPIS_PC_CASE(THREADS, PROD)                                                        \
+  case THREADS * 16 + PROD:                                                                 \
+    return nt ? launch_colgroup_pc_cfg<T, THREADS, PROD, true>(p, x, y, st)                 \
+              : launch_colgroup_pc_cfg<T, THREADS, PROD, false>(p, x, y, st)
+  switch (p->colblock_pc_threads * 16 + p->colblock_pc_prod) {
+    LAPIS_PC_CASE(1024, 4);
+    LAPIS_PC_CASE(1024, 6);
+    LAPIS_PC_CASE(768, 3);
+    LAPIS_PC_CASE(640, 4);
+    LAPIS_PC_CASE(512, 3);
+    LAPIS_PC_CASE(512, 2);
+    default:
+      return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT,
+                       "colblock: no producer/consumer kernel with %d threads and %d producer wavefronts",
+                       p->colblock_pc_threads, p->colblock_pc_prod);
+  }
+#undef LAPIS_PC_CASE
+}
+
 template <typename T>
 int launch_colgroup(const lapis_hip_csr_plan *p, const T *x, T *y, hipStream_t st) {
   if (p->colblock_nunits == 0) return LAPIS_HIP_OK;
+  if (p->colblock_pc_prod > 0) return launch_colgroup_pc<T>(p, x, y, st);
   switch (p->colblock_threads) {
     case 1024: return launch_colgroup_threads<T, 1024>(p, x, y, st);
     case 512: return launch_colgroup_threads<T, 512>(p, x, y, st);
@@ -336,7 +592,7 @@ int build_colgroup(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int 
   T *val_out = nullptr;
   unsigned *idx = nullptr, *perm = nullptr;
   int *tile_ptr = nullptr, *block_range = nullptr, *long_flag = nullptr, *long_rank = nullptr, *long_rows = nullptr,
-      *units = nullptr;
+      *units = nullptr, *fault = nullptr;
   void *scan_temp = nullptr;
   size_t scan_bytes = 0;
   auto release = [&](bool all) {
@@ -353,6 +609,7 @@ int build_colgroup(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int 
       if (tile_ptr) (void)hipFree(tile_ptr);
       if (long_rows) (void)hipFree(long_rows);
       if (units) (void)hipFree(units);
+      if (fault) (void)hipFree(fault);
     }
   };
   auto fail = [&](hipError_t e, const char *what) {
@@ -400,8 +657,13 @@ int build_colgroup(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int 
   // 2. sort the entries by (block, column, row in block)
   const size_t ntiles = (size_t)nblocks * ((size_t)nslices + 1);
   if ((e = hipMalloc(&keys_in, sizeof(unsigned long long) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
-  if ((e = hipMalloc(&val_out, sizeof(T) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
-  if ((e = hipMalloc(&idx, sizeof(unsigned) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
+  // kPcPad entries behind both arrays: the producer wavefronts load whole chunks
+  if ((e = hipMalloc(&val_out, sizeof(T) * ((size_t)nnz + kPcPad))) != hipSuccess) return fail(e, "hipMalloc");
+  if ((e = hipMalloc(&idx, sizeof(unsigned) * ((size_t)nnz + kPcPad))) != hipSuccess) return fail(e, "hipMalloc");
+  if ((e = hipMemsetAsync(val_out + nnz, 0, sizeof(T) * kPcPad, st)) != hipSuccess) return fail(e, "hipMemsetAsync");
+  if ((e = hipMemsetAsync(idx + nnz, 0, sizeof(unsigned) * kPcPad, st)) != hipSuccess) return fail(e, "hipMemsetAsync");
+  if ((e = hipMalloc(&fault, sizeof(int))) != hipSuccess) return fail(e, "hipMalloc");
+  if ((e = hipMemsetAsync(fault, 0, sizeof(int), st)) != hipSuccess) return fail(e, "hipMemsetAsync");
   if ((e = hipMalloc(&tile_ptr, sizeof(int) * ntiles)) != hipSuccess) return fail(e, "hipMalloc");
   if ((e = hipMalloc(&block_range, sizeof(int) * 2 * (size_t)nblocks)) != hipSuccess) return fail(e, "hipMalloc");
   hipLaunchKernelGGL(colgroup_keys_kernel, dim3((unsigned)ceil_div(nrows, 4)), dim3(256), 0, st, (int)nrows, row_bits,
@@ -483,6 +745,20 @@ int build_colgroup(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int 
   p->colblock_epl = env_or("LAPIS_HIP_COLBLOCK_EPL", 8);  // entries per thread and trip
   p->colblock_rows = rows;
   p->colblock_threads = threads;
+  p->colblock_fault = fault;
+  {
+    // Producer and consumer wavefronts: the ring and the tile pointers have to fit beside the row sums,
+    // and a consumer lane finds its slice by walking the tile pointers, which wants tiles of some size.
+    // LAPIS_HIP_COLBLOCK_PC = n > 0 selects the kernel with n producer wavefronts (1024 threads: 4 or
+    // 6; 768: 3; 640: 4; 512: 2 or 3 -- LAPIS_HIP_COLBLOCK_PC_THREADS).  It is not the default: on
+    // MI355X it runs config 2 in 0.294-0.32 ms against 0.305 ms and config 3 in 0.174-0.191 ms against
+    // 0.160 ms for the kernel whose wavefronts do both.
+    int prod = env_or("LAPIS_HIP_COLBLOCK_PC", 0);
+    const int pc_threads = env_or("LAPIS_HIP_COLBLOCK_PC_THREADS", 1024);
+    if (colgroup_pc_lds_bytes(rows, nslices, (int)sizeof(T)) > 160 * 1024) prod = 0;
+    p->colblock_pc_prod = std::max(0, prod);
+    p->colblock_pc_threads = pc_threads;
+  }
   p->colblock_nblocks = nblocks;
   p->colblock_nblocks_nat = nblocks_nat;
   p->colblock_nslices = nslices;

@@ -34,6 +34,9 @@ struct lapis_hip_csr_plan {
   int colblock_rows;         // rows per wavefront (512 or 1024), or per workgroup in the workgroup-blocked layout
   int colblock_threads;      // threads per workgroup of the workgroup-blocked kernel (256, 512 or 1024)
   int colblock_group;        // 1: workgroup-blocked layout (tiles in column order, row sums shared by a workgroup)
+  int colblock_pc_prod;      // > 0: the workgroup kernel with this many producer wavefronts (they only stream)
+  int colblock_pc_threads;   // threads per workgroup of that kernel
+  int *colblock_fault;       // device int: set by a wavefront of that kernel whose bounded wait ran out
   int colblock_nblocks;      // row blocks of the workgroup-blocked layout
   int colblock_nslices;      // slices of x
   int *colblock_tile_ptr;    // device, int[nblocks * (nslices + 1)]

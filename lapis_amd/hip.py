@@ -43,6 +43,12 @@ class CsrStats(ctypes.Structure):
         return d
 
 
+class _CalibrateMode(ctypes.Structure):
+    _fields_ = [(name, ctypes.c_int) for name in (
+        "threads", "workgroups", "stream_in_flight", "gathers_in_flight", "lanes_per_line", "roles", "producers",
+        "stream_behind", "stream_policy", "stream_in_l2", "scalar", "scalar_ahead", "scalar_stride")]
+
+
 _SIGNATURES = {
     "lapis_hip_init": [],
     "lapis_hip_finalize": [],
@@ -52,6 +58,9 @@ _SIGNATURES = {
                                      ctypes.POINTER(_dbl)],
     "lapis_hip_calibrate_gather": [_vp, _i64, _int, _vp, _i64, _i64, _vp, ctypes.POINTER(_dbl), ctypes.POINTER(_dbl),
                                    ctypes.POINTER(_dbl), _vp],
+    "lapis_hip_calibrate_mix": [ctypes.POINTER(_CalibrateMode), _vp, _i64, _vp, _i64, _i64, _i64, _vp, _vp,
+                                ctypes.POINTER(_dbl), ctypes.POINTER(_dbl), ctypes.POINTER(_dbl), ctypes.POINTER(_int),
+                                _vp],
     "lapis_hip_csr_plan_create": [ctypes.POINTER(_vp), _i64, _i64, _i64, _vp, _vp, _int, _vp],
     "lapis_hip_csr_plan_set_kernel": [_vp, _int, _int],
     "lapis_hip_csr_plan_get_stats": [_vp, ctypes.POINTER(CsrStats)],
@@ -59,6 +68,7 @@ _SIGNATURES = {
     "lapis_hip_csr_plan_build_colblock": [_vp, _vp, _vp, _int, _int, _int, _vp],
     "lapis_hip_csr_plan_analyze": [_vp, _vp, _vp, _int, _vp],
     "lapis_hip_csr_plan_update_values": [_vp, _vp, _int, _vp],
+    "lapis_hip_csr_plan_check": [_vp, _vp],
     "lapis_hip_spmv_csr_f64_i32": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp],
     "lapis_hip_spmv_csr_f32_i32": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp],
     "lapis_hip_spmm_csr_f32_i32": [_i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp],
@@ -213,6 +223,11 @@ class CsrPlan:
         check(self._lib.lapis_hip_csr_plan_update_values(self._handle, _ptr(val), val.element_size(), _stream(stream)))
         return self
 
+    def check(self, stream=None):
+        """Wait for the stream and raise if a kernel of this plan gave up a bounded wait between its wavefronts."""
+        check(self._lib.lapis_hip_csr_plan_check(self._handle, _stream(stream)))
+        return self
+
     def destroy(self):
         if self._handle:
             self._lib.lapis_hip_csr_plan_destroy(self._handle)
@@ -281,6 +296,22 @@ def calibrate_gather(x, window_bytes, lanes_per_line, stream_buf, gathers, sink,
                                          gathers, _ptr(sink), ctypes.byref(ms), ctypes.byref(done), ctypes.byref(sbytes),
                                          _stream(stream)))
     return {"ms": ms.value, "gathers": done.value, "stream_bytes": sbytes.value}
+
+
+def calibrate_mix(mode, x, window_bytes, stream_buf, stream_bytes, gathers, cu_count, sink, stream=None):
+    """One arrangement of streaming and gathering wavefronts (lapis_hip_calibrate_mix): ``mode`` is a dict of the
+    fields of lapis_hip_calibrate_mode (missing ones are 0, lanes_per_line 1).  Returns dict(ms, gathers,
+    stream_bytes, cus_with_both_roles)."""
+    lib = init()
+    fn = lib.lapis_hip_calibrate_mix
+    m = _CalibrateMode(**dict({"lanes_per_line": 1}, **mode))
+    ms, done, sbytes, both = _dbl(0.0), _dbl(0.0), _dbl(0.0), _int(-1)
+    check(fn(ctypes.byref(m), _ptr(x) if x is not None else None, window_bytes,
+             _ptr(stream_buf) if stream_buf is not None else None,
+             stream_buf.numel() * stream_buf.element_size() if stream_buf is not None else 0, int(stream_bytes),
+             int(gathers), _ptr(cu_count) if cu_count is not None else None, _ptr(sink), ctypes.byref(ms),
+             ctypes.byref(done), ctypes.byref(sbytes), ctypes.byref(both), _stream(stream)))
+    return {"ms": ms.value, "gathers": done.value, "stream_bytes": sbytes.value, "cus_with_both_roles": both.value}
 
 
 def dot_noalloc(x, y, result, init_value=0.0, stream=None):

@@ -122,11 +122,24 @@ def test_column_blocked_copy_matches_oracle(gpu, cases, slice_log2, layout):
         plan.destroy()
 
 
+# (producer wavefronts, threads per workgroup) of the workgroup kernel; 0 = every wavefront streams and gathers
+ROLE_SPLITS = [(0, 0), (4, 1024), (6, 1024), (3, 768), (4, 640), (2, 512)]
+
+
+def _set_role_split(monkeypatch, split):
+    monkeypatch.setenv("LAPIS_HIP_COLBLOCK_PC", str(split[0]))
+    if split[0]:
+        monkeypatch.setenv("LAPIS_HIP_COLBLOCK_PC_THREADS", str(split[1]))
+
+
+@pytest.mark.parametrize("split", ROLE_SPLITS)
 @pytest.mark.parametrize("long_threshold,unit,rows", [(2, 100, 4096), (64, 5000, 4096), (1024, 0, 8192),
                                                       (100000000, 33333, 16384)])
-def test_workgroup_layout_with_forced_long_rows_and_units(gpu, cases, monkeypatch, long_threshold, unit, rows):
+def test_workgroup_layout_with_forced_long_rows_and_units(gpu, cases, monkeypatch, long_threshold, unit, rows, split):
     # the tuning overrides move rows between their natural blocks and the blocks of long rows
-    # and change how many work units a block is cut into: every combination must give the same y
+    # and change how many work units a block is cut into: every combination must give the same y,
+    # with every wavefront streaming and gathering and with the roles split between wavefronts
+    _set_role_split(monkeypatch, split)
     monkeypatch.setenv("LAPIS_HIP_COLBLOCK_LONG", str(long_threshold))
     monkeypatch.setenv("LAPIS_HIP_COLBLOCK_UNIT", str(unit))
     monkeypatch.setenv("LAPIS_HIP_COLBLOCK_ROWS", str(rows))
@@ -134,7 +147,7 @@ def test_workgroup_layout_with_forced_long_rows_and_units(gpu, cases, monkeypatc
     for name, (A, x, y_in, want, scale) in built.items():
         if A.nnz == 0:
             continue
-        print("case", name, "group", long_threshold, unit, rows, np.dtype(dtype).name, flush=True)
+        print("case", name, "group", long_threshold, unit, rows, split, np.dtype(dtype).name, flush=True)
         pos, crd, val = dev(A.pos), dev(A.crd), dev(A.val)
         plan = gpu.CsrPlan(A.nrows, A.ncols, pos, crd, value_bytes=np.dtype(dtype).itemsize)
         plan.build_colblock(crd, val, 7, layout="group")
@@ -142,10 +155,13 @@ def test_workgroup_layout_with_forced_long_rows_and_units(gpu, cases, monkeypatc
         gpu.spmv(plan, A.nrows, A.ncols, pos, crd, val, dev(x), y)
         torch.cuda.synchronize()
         assert_rows_close(y.cpu().numpy(), want, scale, dtype, "%s/group long>=%d unit %d" % (name, long_threshold, unit))
+        plan.check()
         plan.destroy()
 
 
-def test_workgroup_layout_on_seeded_random_shapes(gpu, oracle, monkeypatch):
+@pytest.mark.parametrize("split", ROLE_SPLITS[:3])
+def test_workgroup_layout_on_seeded_random_shapes(gpu, oracle, monkeypatch, split):
+    _set_role_split(monkeypatch, split)
     # 40 matrices of random shape, density and skew, each with its own slice width, work-unit size,
     # long-row threshold and block size: unit borders fall inside tiles, on tile borders and
     # next to empty tiles
@@ -178,6 +194,7 @@ def test_workgroup_layout_on_seeded_random_shapes(gpu, oracle, monkeypatch):
         gpu.spmv(plan, A.nrows, A.ncols, pos, crd, val, dev(x), y)
         torch.cuda.synchronize()
         assert_rows_close(y.cpu().numpy(), want, scale, dtype, "random case %d" % case)
+        plan.check()
         plan.destroy()
 
 
