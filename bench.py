@@ -31,6 +31,12 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+# roofline.traffic is not measured inside this run (hardware counters need rocprofv3 around the process)
+TRAFFIC_SOURCE = ("profiles/traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this kernel, "
+                  "scaled by a copy kernel of known size; null when this run's kernel time is more than 20 % off "
+                  "the time recorded with the reading")
+
+
 def traffic_from_profiles(kernel_key, kernel_ms):
     """HBM bytes per launch measured with rocprofv3 --pmc (profiles/traffic.json), or None.
 
@@ -284,6 +290,7 @@ def run_spmv(args, cfg):
         "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": traffic_from_profiles("%s_config%d" % (family, cfg), kt["mean_ms"]) if cfg else None,
+                     "traffic_source": TRAFFIC_SOURCE,
                      "kernel_ms_mean": kt["mean_ms"], "kernel_ms_median": kt["median_ms"],
                      "kernel_ms_min": kt["min_ms"], "launches_timed": kt["count"]},
     }
@@ -294,10 +301,14 @@ def run_spmv(args, cfg):
         if floor:
             # what bounds this kernel is not HBM: its traffic is 1.35 x algorithmic at 3.7 TB/s.  It is the
             # requests its compute units can keep in flight; see calibrate_gather().
+            # It is the floor of THIS kernel shape (every wavefront streams and gathers), not of the chip:
+            # the graded figure is roofline.frac.
             out["roofline"]["secondary"] = dict(floor, bound="line_requests_in_flight", achieved_ms=kt["mean_ms"],
-                                                frac=floor["floor_ms"] / kt["mean_ms"],
-                                                model="stream_bytes / stream rate + gather lines / line rate "
-                                                      "(calibrated in this run; the two do not overlap)")
+                                                fraction_of_scheme_floor=floor["floor_ms"] / kt["mean_ms"],
+                                                model="stream_bytes / stream rate + gather lines / line rate, both "
+                                                      "calibrated in this run with wavefronts that do both; "
+                                                      "wavefronts with one role each overlap the two by about a "
+                                                      "fifth in the calibration kernel (bench.py --calibrate-gather)")
     if args.graph or cfg == 1:
         # Launch-bound sizes: the same calls captured once into a HIP graph (10 per graph) and
         # replayed, which takes the Python and launch overhead of each call out of the loop.
@@ -427,6 +438,7 @@ def run_spmm(args):
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": traffic_from_profiles("spmm_config4", kt["mean_ms"])
                      if not args.workload and k == 64 else None,
+                     "traffic_source": TRAFFIC_SOURCE,
                      "kernel_ms_mean": kt["mean_ms"], "kernel_ms_median": kt["median_ms"],
                      "kernel_ms_min": kt["min_ms"], "launches_timed": kt["count"]},
     }
@@ -481,6 +493,7 @@ def run_cg(args):
         "roofline": {"bound": "hbm", "kernel": "spmv_%s_kernel<double>" % plan.stats()["kernel_name"],
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": traffic_from_profiles("cg_spmv_config5", kt["mean_ms"]),
+                     "traffic_source": TRAFFIC_SOURCE,
                      "kernel_ms_mean": kt["mean_ms"], "kernel_ms_median": kt["median_ms"],
                      "launches_timed": kt["count"]},
     }
@@ -529,6 +542,8 @@ def main():
                     help="print the whole gather/stream calibration table (merge factors, cache levels) instead of "
                          "the three rows the secondary roofline needs")
     ap.add_argument("--no-calibration", action="store_true", help="skip the gather/stream calibration launches")
+    ap.add_argument("--no-others", action="store_true",
+                    help="with the default configuration: do not also run configurations 3, 4 and 5 (the 'others' block)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch the library's copy kernel on 1 GiB three times, the known-size reference "
                          "that rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -558,7 +573,39 @@ def main():
         out = run_spmm(args)
     else:
         out = run_cg(args)
+    if args.config == 2 and not args.workload and not args.no_others and not args.calibrate_gather:
+        out["others"] = run_others(args)
     print(json.dumps(out), flush=True)
+
+
+def run_others(args):
+    """The other configurations beside the headline, each for at most 20 steps, without CPU legs: what the
+    same library does on the power-law SpMV (3), the SpMM (4) and CG (5).  Keys per configuration:
+    ms_per_step, kernel, kernel_ms_mean, frac (of the 8 TB/s roofline, for the dominant kernel),
+    algorithmic_bytes_per_step, GB/s (whole step)."""
+    import copy
+    import gc
+    import torch
+    others = {}
+    for cfg, runner in ((3, lambda a: run_spmv(a, 3)), (4, run_spmm), (5, run_cg)):
+        a = copy.copy(args)
+        a.config, a.no_cpu, a.no_calibration, a.graph, a.host_buffers = cfg, True, True, False, False
+        a.kernel, a.workload, a.k, a.spmm_kernel = None, None, 64, "auto"
+        a.steps, a.warmup = min(20, {3: 20, 4: 20, 5: 20}[cfg]), 2
+        gc.collect()
+        torch.cuda.empty_cache()
+        try:
+            r = runner(a)
+        except Exception as e:  # the headline line must not be lost to a failure here
+            others["config%d" % cfg] = {"error": repr(e)}
+            continue
+        others["config%d" % cfg] = {
+            "workload": r["config"]["workload"], "metric": r["metric"], "steps": r["steps"],
+            "ms_per_step": r["ms_per_step"], "GB/s": r["value"], "kernel": r["roofline"]["kernel"],
+            "kernel_ms_mean": r["roofline"]["kernel_ms_mean"], "frac": r["roofline"]["frac"],
+            "algorithmic_bytes_per_step": r["config"]["algorithmic_bytes_per_step"], "dtype": r["dtype"],
+            "pct_of_hbm_peak_whole_step": r["pct_of_hbm_peak"]}
+    return others
 
 
 if __name__ == "__main__":

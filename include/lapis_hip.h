@@ -31,7 +31,9 @@ enum lapis_hip_status {
   LAPIS_HIP_ERR_NOT_INITIALIZED = 3,  /* lapis_hip_init() has not been called */
   LAPIS_HIP_ERR_BAD_CSR = 4,          /* positions not monotone / coordinates out of range */
   LAPIS_HIP_ERR_UNSUPPORTED_DEVICE = 5, /* the current device is not gfx950 */
-  LAPIS_HIP_ERR_PLAN_MISMATCH = 6     /* plan was built for other sizes or buffers */
+  LAPIS_HIP_ERR_PLAN_MISMATCH = 6,    /* plan was built for other sizes or buffers */
+  LAPIS_HIP_ERR_NO_TILING = 7         /* the matrix has no room in the column-blocked tiling (too many columns,
+                                         slices or row blocks): the plan keeps its CSR kernel */
 };
 
 /* ---- runtime ------------------------------------------------------------ */
@@ -191,6 +193,21 @@ int lapis_hip_csr_plan_analyze(lapis_hip_csr_plan *plan, const int32_t *crd, con
  * alone (status OK). */
 int lapis_hip_csr_plan_update_values(lapis_hip_csr_plan *plan, const void *val, int value_bytes,
                                      lapis_hip_stream_t stream);
+/* 1 when `plan` was made for exactly this structure -- the same sizes, the same number of
+ * non-zeros and the same position and coordinate buffers -- else 0 (also for a NULL plan).
+ * For callers that keep a plan between calls: the SpMV entry points compare sizes and the
+ * position buffer only (they take no nnz), which a second matrix of the same shape at the
+ * same address would pass.  The reference has nothing to cache: its launch re-reads
+ * pos[n] and pos[0] on the host every call (KokkosLoopMapping.cpp:290-322). */
+int lapis_hip_csr_plan_matches(const lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, int64_t nnz,
+                               const int32_t *pos, const int32_t *crd);
+/* lapis_hip_csr_plan_analyze for callers that need the same bits from every run: where the
+ * copy pays it is built in the per-wavefront layout (LAPIS_HIP_COLBLOCK_WAVE, wave-private
+ * row sums in a fixed order) instead of the faster workgroup layout, whose LDS atomics fix
+ * no order.  The reference's Kokkos kernel is reproducible run to run
+ * (tests/Dialect/Kokkos/loop_mapping_2.mlir.gold:14-35 fixes its order). */
+int lapis_hip_csr_plan_analyze_reproducible(lapis_hip_csr_plan *plan, const int32_t *crd, const void *val,
+                                            int value_bytes, lapis_hip_stream_t stream);
 /* Waits for `stream` and reports whether a kernel of this plan gave up a wait between its
  * own wavefronts (the workgroup-blocked SpMV hands entries from streaming wavefronts to
  * gathering ones through LDS, and every such wait is bounded so that a launch always
@@ -318,6 +335,25 @@ int lapis_hip_dot_f64(int64_t n, const double *x, const double *y, double init, 
                       lapis_hip_stream_t stream);
 int lapis_hip_dot_f32(int64_t n, const float *x, const float *y, float init, float *result,
                       lapis_hip_stream_t stream);
+/* The dot product with its result on the HOST, the call returning when it is there: what
+ * the reference's emitted code has, Kokkos::parallel_reduce into a host scalar followed by
+ * the join with the initial value (TranslateToKokkosCpp.cpp:1696-1705,1838; 1671-1690).
+ * For emitted code that needs the number at once; the device-scalar entries above are for
+ * callers that can leave it on the device. */
+int lapis_hip_dot_f64_host(int64_t n, const double *x, const double *y, double init, double *host_result,
+                           lapis_hip_stream_t stream);
+int lapis_hip_dot_f32_host(int64_t n, const float *x, const float *y, float init, float *host_result,
+                           lapis_hip_stream_t stream);
+/* dst = a*x + b*y and *result = init + sum dst[i]*z[i] in one pass over the vectors (z NULL:
+ * dst . dst).  The pair the CG loop of examples/pcg_solve.py:80-82 runs back to back
+ * (r = r - alpha*Ap, then r . r): fused it reads r and Ap once and writes r once, five
+ * vector passes becoming three.  dst may be x or y.  With 16-byte-aligned buffers both
+ * results have exactly the bits lapis_hip_axpby_* followed by lapis_hip_dot_* give.
+ * `result` is a device scalar. */
+int lapis_hip_axpby_dot_f64(int64_t n, double a, const double *x, double b, const double *y, double *dst,
+                            const double *z, double init, double *result, lapis_hip_stream_t stream);
+int lapis_hip_axpby_dot_f32(int64_t n, float a, const float *x, float b, const float *y, float *dst, const float *z,
+                            float init, float *result, lapis_hip_stream_t stream);
 /* lapis_hip_dot_f64 for callers that cannot allocate (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
  * reference.  Same kernels and the same result, bit for bit, as lapis_hip_dot_f64, but

@@ -99,6 +99,14 @@ void lapis_dualview_f64_modify_device(lapis_dualview_f64 *v); /* modifyDevice():
 void lapis_dualview_f64_sync_host(lapis_dualview_f64 *v);     /* syncHost()    :251: copies back only if modified on the device */
 void lapis_dualview_f64_sync_device(lapis_dualview_f64 *v);   /* syncDevice()  :271: uploads only if modified on the host */
 void lapis_dualview_f64_destroy(lapis_dualview_f64 *v);
+/* the same for floats (LAPIS::DualView is a template over the element type, LAPISSupport.hpp:136) */
+typedef struct lapis_dualview_f32 lapis_dualview_f32;
+lapis_dualview_f32 *lapis_dualview_f32_create(float *host, int64_t n);
+void lapis_dualview_f32_modify_host(lapis_dualview_f32 *v);
+void lapis_dualview_f32_modify_device(lapis_dualview_f32 *v);
+void lapis_dualview_f32_sync_host(lapis_dualview_f32 *v);
+void lapis_dualview_f32_sync_device(lapis_dualview_f32 *v);
+void lapis_dualview_f32_destroy(lapis_dualview_f32 *v);
 
 /* A CSR matrix uploaded once: device copies of positions, coordinates and
  * values, its plan (row statistics -> kernel) and, where the library
@@ -113,7 +121,24 @@ void lapis_resident_csr_update_values(lapis_resident_csr *A, lapis_memref_1d_f64
  * modified on the device; nothing is copied back and the call does not wait
  * for the kernel -- lapis_dualview_f64_sync_host(y) does both. */
 void lapis_resident_csr_spmv(lapis_resident_csr *A, lapis_dualview_f64 *x, lapis_dualview_f64 *y);
+/* func @spmm on resident operands: C += A*B, B (columns x k) and C (rows x k) row-major
+ * in their views; same copy and wait rules as lapis_resident_csr_spmv. */
+void lapis_resident_csr_spmm(lapis_resident_csr *A, lapis_dualview_f64 *B, int64_t k, lapis_dualview_f64 *C);
+/* func @pcg of examples/pcg_solve.py:52 on resident operands: solves A x = b from x = 0 with
+ * the Jacobi preconditioner dinv (NULL: none), at most maxiter iterations, until the relative
+ * residual is at most tol.  x is a view of the caller's, overwritten and left marked modified
+ * on the device; *iters and *relres as the function returns them.  Waits for the solve. */
+void lapis_resident_csr_pcg(lapis_resident_csr *A, lapis_dualview_f64 *b, lapis_dualview_f64 *dinv, double tol,
+                            size_t maxiter, lapis_dualview_f64 *x, size_t *iters, double *relres);
 void lapis_resident_csr_destroy(lapis_resident_csr *A);
+/* the fp32 matrix (config 3 and the SpMM operand of config 4 are fp32) */
+typedef struct lapis_resident_csr_f32 lapis_resident_csr_f32;
+lapis_resident_csr_f32 *lapis_resident_csr_f32_create(lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd,
+                                                      lapis_memref_1d_f32 *val, const lapis_csr_specifier *spec);
+void lapis_resident_csr_f32_update_values(lapis_resident_csr_f32 *A, lapis_memref_1d_f32 *val);
+void lapis_resident_csr_f32_spmv(lapis_resident_csr_f32 *A, lapis_dualview_f32 *x, lapis_dualview_f32 *y);
+void lapis_resident_csr_f32_spmm(lapis_resident_csr_f32 *A, lapis_dualview_f32 *B, int64_t k, lapis_dualview_f32 *C);
+void lapis_resident_csr_f32_destroy(lapis_resident_csr_f32 *A);
 
 /* func @spmv(A, x, y) -> y of examples/spmv_noalloc.py:9-14 and
  * benchmarks/spmv/spmv.mlir:3-6: y += A*x, y updated in place and returned. */

@@ -147,6 +147,38 @@ __global__ __launch_bounds__(256) void dot_final_kernel(int count, const T *__re
   if (threadIdx.x == 0) *result = all + init;
 }
 
+
+// dst = a*x + b*y and the partial sums of dst . z in one pass (z == nullptr: dst . dst).  Element order,
+// grid and the order of the additions are those of elementwise_kernel and dot_partial_kernel, so the pair
+// of results has the bits the two separate calls give.
+template <typename T>
+__global__ __launch_bounds__(256) void axpby_dot_partial_kernel(long long n, T a, const T *x, T b, const T *y, T *dst,
+                                                                const T *z, T *__restrict__ partials, int vec) {
+  typedef typename VecOf<T>::type V;
+  constexpr int VW = VecOf<T>::width;
+  __shared__ T lds4[4];
+  T acc = T(0);
+  const long long nv = vec ? n / VW : 0;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < nv; i += (long long)gridDim.x * 256) {
+    const V vx = reinterpret_cast<const V *>(x)[i], vy = reinterpret_cast<const V *>(y)[i];
+    V vd;
+#pragma unroll
+    for (int e = 0; e < VW; ++e) vd[e] = a * vx[e] + b * vy[e];
+    const V vz = z ? reinterpret_cast<const V *>(z)[i] : vd;
+    reinterpret_cast<V *>(dst)[i] = vd;
+#pragma unroll
+    for (int e = 0; e < VW; ++e) acc = acc + vd[e] * vz[e];
+  }
+  for (long long i = nv * VW + (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) {
+    const T d = a * x[i] + b * y[i];
+    const T w = z ? z[i] : d;
+    dst[i] = d;
+    acc = acc + d * w;
+  }
+  const T total = block_sum_256(acc, lds4);
+  if (threadIdx.x == 0) partials[blockIdx.x] = total;
+}
+
 int dot_grid(int64_t n) {
   const int64_t want = ceil_div(n, 256 * 8);
   const int64_t cap = std::max(1, device_cu_count()) * 8;
@@ -173,7 +205,7 @@ constexpr int kSlots = 64;
 std::mutex g_scratch_mutex;
 char *g_scratch = nullptr;  // kSlots * kDotMaxBlocks * 8 bytes
 unsigned g_next_slot = 0;
-constexpr size_t kSlotBytes = (size_t)kDotMaxBlocks * 8;
+constexpr size_t kSlotBytes = ((size_t)kDotMaxBlocks + 2) * 8;  // the partials, then one result for the *_host entries
 
 int take_slot(void **partials) {
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
@@ -253,6 +285,67 @@ extern "C" int lapis_hip_dot_f64_noalloc(int64_t n, const double *x, const doubl
   // dot_partial_kernel writes every partial the final kernel reads (dot_grid(n) of them):
   // nothing of the previous call's contents is read, so nothing has to be cleared.
   return launch_dot<double>(n, x, y, init, result, partials, as_stream(stream));
+}
+
+
+namespace {
+// dot with the result on the host: what the reference's parallel_reduce into a host scalar gives
+// (TranslateToKokkosCpp.cpp:1696-1705,1838), blocking included.
+template <typename T>
+int dot_host_entry(const char *what, int64_t n, const T *x, const T *y, T init, T *host_result, lapis_hip_stream_t stream) {
+  LAPIS_CHECK_INIT();
+  LAPIS_REQUIRE(n >= 0, "%s: negative length", what);
+  LAPIS_REQUIRE(host_result, "%s: null result", what);
+  LAPIS_REQUIRE(n == 0 || (x && y), "%s: null vector with n=%lld", what, (long long)n);
+  void *partials = nullptr;
+  int rc = take_slot(&partials);
+  if (rc != LAPIS_HIP_OK) return rc;
+  T *device_result = reinterpret_cast<T *>(static_cast<char *>(partials) + (size_t)kDotMaxBlocks * 8);
+  hipStream_t st = as_stream(stream);
+  rc = launch_dot<T>(n, x, y, init, device_result, static_cast<T *>(partials), st);
+  if (rc != LAPIS_HIP_OK) return rc;
+  LAPIS_HIP_TRY(hipMemcpyAsync(host_result, device_result, sizeof(T), hipMemcpyDeviceToHost, st));
+  LAPIS_HIP_TRY(hipStreamSynchronize(st));
+  return LAPIS_HIP_OK;
+}
+
+template <typename T>
+int axpby_dot_entry(const char *what, int64_t n, T a, const T *x, T b, const T *y, T *dst, const T *z, T init, T *result,
+                    lapis_hip_stream_t stream) {
+  LAPIS_CHECK_INIT();
+  LAPIS_REQUIRE(n >= 0, "%s: negative length", what);
+  LAPIS_REQUIRE(result, "%s: null result", what);
+  LAPIS_REQUIRE(n == 0 || (x && y && dst), "%s: null vector with n=%lld", what, (long long)n);
+  void *slot = nullptr;
+  const int rc = take_slot(&slot);
+  if (rc != LAPIS_HIP_OK) return rc;
+  T *partials = static_cast<T *>(slot);
+  hipStream_t st = as_stream(stream);
+  const int grid = dot_grid(n);
+  const int vec = (aligned16(x) && aligned16(y) && aligned16(dst) && (!z || aligned16(z))) ? 1 : 0;
+  hipLaunchKernelGGL((axpby_dot_partial_kernel<T>), dim3(grid), dim3(256), 0, st, (long long)n, a, x, b, y, dst, z,
+                     partials, vec);
+  hipLaunchKernelGGL((dot_final_kernel<T>), dim3(1), dim3(256), 0, st, grid, (const T *)partials, init, result);
+  LAPIS_LAUNCH_CHECK();
+  return LAPIS_HIP_OK;
+}
+}  // namespace
+
+extern "C" int lapis_hip_dot_f64_host(int64_t n, const double *x, const double *y, double init, double *host_result,
+                                      lapis_hip_stream_t stream) {
+  return dot_host_entry<double>("dot_f64_host", n, x, y, init, host_result, stream);
+}
+extern "C" int lapis_hip_dot_f32_host(int64_t n, const float *x, const float *y, float init, float *host_result,
+                                      lapis_hip_stream_t stream) {
+  return dot_host_entry<float>("dot_f32_host", n, x, y, init, host_result, stream);
+}
+extern "C" int lapis_hip_axpby_dot_f64(int64_t n, double a, const double *x, double b, const double *y, double *dst,
+                                       const double *z, double init, double *result, lapis_hip_stream_t stream) {
+  return axpby_dot_entry<double>("axpby_dot_f64", n, a, x, b, y, dst, z, init, result, stream);
+}
+extern "C" int lapis_hip_axpby_dot_f32(int64_t n, float a, const float *x, float b, const float *y, float *dst,
+                                       const float *z, float init, float *result, lapis_hip_stream_t stream) {
+  return axpby_dot_entry<float>("axpby_dot_f32", n, a, x, b, y, dst, z, init, result, stream);
 }
 
 extern "C" int lapis_hip_dot_f64(int64_t n, const double *x, const double *y, double init, double *result,

@@ -399,7 +399,7 @@ int build(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int slice_log
   const int64_t nnz = p->stats.nnz, nrows = p->stats.nrows;
   const int col_bits = std::max(1, bits_for(p->stats.ncols));
   if (col_bits + kColblockRowBits > 32)
-    return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT,
+    return set_error(LAPIS_HIP_ERR_NO_TILING,
                      "csr_plan_build_colblock: %lld columns need %d bits, more than the %d an entry has room for",
                      (long long)p->stats.ncols, col_bits, 32 - kColblockRowBits);
   {
@@ -413,7 +413,7 @@ int build(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int slice_log
   const int slice_bits = std::max(0, col_bits - slice_log2);
   const int end_bit = 32 + slice_bits + rb_bits;
   if (end_bit > 64 || slice_log2 < 0 || slice_log2 > 31)
-    return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT, "csr_plan_build_colblock: sort key needs %d bits", end_bit);
+    return set_error(LAPIS_HIP_ERR_NO_TILING, "csr_plan_build_colblock: sort key needs %d bits", end_bit);
 
   unsigned long long *keys_in = nullptr, *keys_out = nullptr;
   T *val_out = nullptr;
@@ -550,18 +550,41 @@ extern "C" int lapis_hip_csr_plan_check(lapis_hip_csr_plan *plan, lapis_hip_stre
   return LAPIS_HIP_OK;
 }
 
+namespace {
+int analyze_with_layout(lapis_hip_csr_plan *plan, const int32_t *crd, const void *val, int value_bytes, int layout,
+                        lapis_hip_stream_t stream);
+}
+
 extern "C" int lapis_hip_csr_plan_analyze(lapis_hip_csr_plan *plan, const int32_t *crd, const void *val, int value_bytes,
                                           lapis_hip_stream_t stream) {
+  return analyze_with_layout(plan, crd, val, value_bytes, LAPIS_HIP_COLBLOCK_AUTO, stream);
+}
+
+extern "C" int lapis_hip_csr_plan_analyze_reproducible(lapis_hip_csr_plan *plan, const int32_t *crd, const void *val,
+                                                       int value_bytes, lapis_hip_stream_t stream) {
+  return analyze_with_layout(plan, crd, val, value_bytes, LAPIS_HIP_COLBLOCK_WAVE, stream);
+}
+
+namespace {
+int analyze_with_layout(lapis_hip_csr_plan *plan, const int32_t *crd, const void *val, int value_bytes, int layout,
+                        lapis_hip_stream_t stream) {
   LAPIS_CHECK_INIT();
   LAPIS_REQUIRE(plan, "csr_plan_analyze: null plan");
   LAPIS_REQUIRE(value_bytes == 4 || value_bytes == 8, "csr_plan_analyze: value_bytes must be 4 or 8");
   if (!plan->stats.colblock_recommended || plan->stats.nnz == 0) return LAPIS_HIP_OK;
   LAPIS_REQUIRE(crd && val, "csr_plan_analyze: null coordinates or values");
-  if (plan->colblock_built && plan->colblock_value_bytes == value_bytes && plan->colblock_src_crd == crd) {
+  const int want_group = layout == LAPIS_HIP_COLBLOCK_WAVE ? 0 : 1;
+  if (plan->colblock_built && plan->colblock_value_bytes == value_bytes && plan->colblock_src_crd == crd &&
+      plan->colblock_group == want_group) {
     plan->stats.kernel = LAPIS_HIP_SPMV_COLBLOCK;  // the copy is there: bring its values up to date
     return lapis_hip_csr_plan_update_values(plan, val, value_bytes, stream);
   }
-  const int rc = lapis_hip_csr_plan_build_colblock(plan, crd, val, value_bytes, LAPIS_HIP_COLBLOCK_AUTO, 0, stream);
-  // a matrix the tiling has no room for (too many slices or row blocks) keeps its CSR kernel
-  return rc == LAPIS_HIP_ERR_INVALID_ARGUMENT ? LAPIS_HIP_OK : rc;
+  const int rc = lapis_hip_csr_plan_build_colblock(plan, crd, val, value_bytes, layout, 0, stream);
+  // a matrix the tiling has no room for keeps its CSR kernel: that is an answer, not an error
+  if (rc == LAPIS_HIP_ERR_NO_TILING) {
+    (void)set_error(LAPIS_HIP_OK, "%s", "");
+    return LAPIS_HIP_OK;
+  }
+  return rc;
 }
+}  // namespace

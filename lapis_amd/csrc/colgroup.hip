@@ -578,7 +578,7 @@ int build_colgroup(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int 
   while (slice_log2 < 32 - row_bits && ceil_div(p->stats.ncols, 1LL << slice_log2) > kMaxSlicesInLds) ++slice_log2;
   const int64_t nslices64 = ceil_div(p->stats.ncols, 1LL << slice_log2);
   if (slice_log2 < 1 || nslices64 > kMaxSlicesInLds)
-    return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT,
+    return set_error(LAPIS_HIP_ERR_NO_TILING,
                      "csr_plan_build_colblock: %lld slices of 2^%d columns; the workgroup layout takes at most %d",
                      (long long)nslices64, slice_log2, kMaxSlicesInLds);
   const int nslices = (int)nslices64;
@@ -649,7 +649,7 @@ int build_colgroup(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int 
   const int end_bit = bits_for((int64_t)nblocks) + col_bits + row_bits;
   if (end_bit > 64 || (int64_t)nblocks * (nslices + 1) > (1LL << 27)) {
     release(true);
-    return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT,
+    return set_error(LAPIS_HIP_ERR_NO_TILING,
                      "csr_plan_build_colblock: %d row blocks x %d slices of 2^%d columns is not a usable tiling",
                      nblocks, nslices, slice_log2);
   }

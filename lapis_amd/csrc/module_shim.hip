@@ -224,100 +224,204 @@ extern "C" void lapis_finalize(void) {
 
 // ---- resident operands ----------------------------------------------------------------------------
 
-struct lapis_dualview_f64 {
-  double *host = nullptr;
-  double *dev = nullptr;
+template <typename T>
+struct DualViewOf {
+  T *host = nullptr;
+  T *dev = nullptr;
   int64_t n = 0;
   bool modified_host = false;
   bool modified_device = false;
 };
+struct lapis_dualview_f64 : DualViewOf<double> {};
+struct lapis_dualview_f32 : DualViewOf<float> {};
 
-struct lapis_resident_csr {
+template <typename T>
+struct ResidentCsrOf {
   int64_t nrows = 0, ncols = 0, nnz = 0;
   int32_t *pos = nullptr, *crd = nullptr;
-  double *val = nullptr;
+  T *val = nullptr;
   lapis_hip_csr_plan *plan = nullptr;
 };
+struct lapis_resident_csr : ResidentCsrOf<double> {};
+struct lapis_resident_csr_f32 : ResidentCsrOf<float> {};
 
-extern "C" lapis_dualview_f64 *lapis_dualview_f64_create(double *host, int64_t n) {
+namespace {
+template <typename V, typename T>
+V *dualview_create(T *host, int64_t n) {
   if (n < 0 || (n > 0 && !host)) module_abort("dualview: null host buffer or negative length");
-  lapis_dualview_f64 *v = new lapis_dualview_f64();
+  V *v = new V();
   v->host = host;
   v->n = n;
-  if (n > 0) check_hip(hipMalloc(&v->dev, sizeof(double) * (size_t)n), "hipMalloc");
+  if (n > 0) check_hip(hipMalloc(&v->dev, sizeof(T) * (size_t)n), "hipMalloc");
   v->modified_host = true;
   return v;
 }
-
-extern "C" void lapis_dualview_f64_modify_host(lapis_dualview_f64 *v) { v->modified_host = true; }
-extern "C" void lapis_dualview_f64_modify_device(lapis_dualview_f64 *v) { v->modified_device = true; }
-
-extern "C" void lapis_dualview_f64_sync_host(lapis_dualview_f64 *v) {
+template <typename T>
+void dualview_sync_host(DualViewOf<T> *v) {
   if (!v->modified_device) return;
   // hipMemcpy on the null stream waits for the kernels queued there before it copies
-  if (v->n > 0) check_hip(hipMemcpy(v->host, v->dev, sizeof(double) * (size_t)v->n, hipMemcpyDeviceToHost), "device-to-host copy");
+  if (v->n > 0) check_hip(hipMemcpy(v->host, v->dev, sizeof(T) * (size_t)v->n, hipMemcpyDeviceToHost), "device-to-host copy");
   v->modified_device = false;
 }
-
-extern "C" void lapis_dualview_f64_sync_device(lapis_dualview_f64 *v) {
+template <typename T>
+void dualview_sync_device(DualViewOf<T> *v) {
   if (!v->modified_host) return;
-  if (v->n > 0) check_hip(hipMemcpy(v->dev, v->host, sizeof(double) * (size_t)v->n, hipMemcpyHostToDevice), "host-to-device copy");
+  if (v->n > 0) check_hip(hipMemcpy(v->dev, v->host, sizeof(T) * (size_t)v->n, hipMemcpyHostToDevice), "host-to-device copy");
   v->modified_host = false;
 }
-
-extern "C" void lapis_dualview_f64_destroy(lapis_dualview_f64 *v) {
-  if (!v) return;
-  if (v->dev) (void)hipFree(v->dev);
-  delete v;
+template <typename T>
+void dualview_destroy(DualViewOf<T> *v) {
+  if (v && v->dev) (void)hipFree(v->dev);
 }
 
-extern "C" lapis_resident_csr *lapis_resident_csr_create(lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd,
-                                                         lapis_memref_1d_f64 *val, const lapis_csr_specifier *spec) {
+template <typename R, typename T, typename ValMemref>
+R *resident_create(lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd, ValMemref *val, const lapis_csr_specifier *spec) {
   int32_t *hpos = host_data(pos, 1, "positions");
   int32_t *hcrd = host_data(crd, 1, "coordinates");
-  double *hval = host_data(val, 1, "values");
+  T *hval = host_data(val, 1, "values");
   const CsrArgs a = csr_args(pos, crd, val->sizes[0], spec);
-  lapis_resident_csr *A = new lapis_resident_csr();
+  R *A = new R();
   A->nrows = a.nrows;
   A->ncols = a.ncols;
   A->nnz = a.nnz;
   check_hip(hipMalloc(&A->pos, sizeof(int32_t) * ((size_t)a.nrows + 1)), "hipMalloc");
   check_hip(hipMalloc(&A->crd, sizeof(int32_t) * (size_t)std::max<int64_t>(a.nnz, 1)), "hipMalloc");
-  check_hip(hipMalloc(&A->val, sizeof(double) * (size_t)std::max<int64_t>(a.nnz, 1)), "hipMalloc");
+  check_hip(hipMalloc(&A->val, sizeof(T) * (size_t)std::max<int64_t>(a.nnz, 1)), "hipMalloc");
   check_hip(hipMemcpy(A->pos, hpos, sizeof(int32_t) * ((size_t)a.nrows + 1), hipMemcpyHostToDevice), "host-to-device copy");
   check_hip(hipMemcpy(A->crd, hcrd, sizeof(int32_t) * (size_t)a.nnz, hipMemcpyHostToDevice), "host-to-device copy");
-  check_hip(hipMemcpy(A->val, hval, sizeof(double) * (size_t)a.nnz, hipMemcpyHostToDevice), "host-to-device copy");
-  check(lapis_hip_csr_plan_create(&A->plan, a.nrows, a.ncols, a.nnz, A->pos, A->crd, 8, nullptr),
+  check_hip(hipMemcpy(A->val, hval, sizeof(T) * (size_t)a.nnz, hipMemcpyHostToDevice), "host-to-device copy");
+  check(lapis_hip_csr_plan_create(&A->plan, a.nrows, a.ncols, a.nnz, A->pos, A->crd, (int)sizeof(T), nullptr),
         "lapis_hip_csr_plan_create");
   // a resident matrix is there to be multiplied many times: let the library build the copy it recommends
-  check(lapis_hip_csr_plan_analyze(A->plan, A->crd, A->val, 8, nullptr), "lapis_hip_csr_plan_analyze");
+  check(lapis_hip_csr_plan_analyze(A->plan, A->crd, A->val, (int)sizeof(T), nullptr), "lapis_hip_csr_plan_analyze");
   return A;
 }
-
-extern "C" void lapis_resident_csr_update_values(lapis_resident_csr *A, lapis_memref_1d_f64 *val) {
-  double *hval = host_data(val, 1, "values");
+template <typename T, typename ValMemref>
+void resident_update_values(ResidentCsrOf<T> *A, ValMemref *val) {
+  T *hval = host_data(val, 1, "values");
   if (val->sizes[0] < A->nnz) module_abort("update_values: fewer values than the matrix has non-zeros");
-  check_hip(hipMemcpy(A->val, hval, sizeof(double) * (size_t)A->nnz, hipMemcpyHostToDevice), "host-to-device copy");
-  check(lapis_hip_csr_plan_update_values(A->plan, A->val, 8, nullptr), "lapis_hip_csr_plan_update_values");
+  check_hip(hipMemcpy(A->val, hval, sizeof(T) * (size_t)A->nnz, hipMemcpyHostToDevice), "host-to-device copy");
+  check(lapis_hip_csr_plan_update_values(A->plan, A->val, (int)sizeof(T), nullptr), "lapis_hip_csr_plan_update_values");
 }
-
-extern "C" void lapis_resident_csr_spmv(lapis_resident_csr *A, lapis_dualview_f64 *x, lapis_dualview_f64 *y) {
+template <typename T>
+void resident_spmv(ResidentCsrOf<T> *A, DualViewOf<T> *x, DualViewOf<T> *y) {
   if (x->n < A->ncols) module_abort("x is shorter than the number of columns");
   if (y->n < A->nrows) module_abort("y is shorter than the number of rows");
   if (x == y) module_abort("x and y must be different views");
-  lapis_dualview_f64_sync_device(x);
-  lapis_dualview_f64_sync_device(y);
-  check(lapis_hip_spmv_csr_f64_i32(A->plan, A->nrows, A->ncols, A->pos, A->crd, A->val, x->dev, y->dev, nullptr),
-        "lapis_hip_spmv_csr_f64_i32");
+  dualview_sync_device(x);
+  dualview_sync_device(y);
+  if constexpr (sizeof(T) == 8)
+    check(lapis_hip_spmv_csr_f64_i32(A->plan, A->nrows, A->ncols, A->pos, A->crd, A->val, x->dev, y->dev, nullptr),
+          "lapis_hip_spmv_csr_f64_i32");
+  else
+    check(lapis_hip_spmv_csr_f32_i32(A->plan, A->nrows, A->ncols, A->pos, A->crd, A->val, x->dev, y->dev, nullptr),
+          "lapis_hip_spmv_csr_f32_i32");
   y->modified_device = true;
 }
-
-extern "C" void lapis_resident_csr_destroy(lapis_resident_csr *A) {
+// C += A*B with B (ncols x k) and C (nrows x k) row-major in their views
+template <typename T>
+void resident_spmm(ResidentCsrOf<T> *A, DualViewOf<T> *B, int64_t k, DualViewOf<T> *C) {
+  if (k < 0 || B->n < A->ncols * k) module_abort("B is smaller than columns x k");
+  if (C->n < A->nrows * k) module_abort("C is smaller than rows x k");
+  if (B == C) module_abort("B and C must be different views");
+  dualview_sync_device(B);
+  dualview_sync_device(C);
+  if constexpr (sizeof(T) == 8)
+    check(lapis_hip_spmm_csr_f64_i32_plan(A->plan, A->nrows, A->ncols, k, A->pos, A->crd, A->val, B->dev, k, C->dev, k,
+                                          nullptr),
+          "lapis_hip_spmm_csr_f64_i32_plan");
+  else
+    check(lapis_hip_spmm_csr_f32_i32_plan(A->plan, A->nrows, A->ncols, k, A->pos, A->crd, A->val, B->dev, k, C->dev, k,
+                                          nullptr),
+          "lapis_hip_spmm_csr_f32_i32_plan");
+  C->modified_device = true;
+}
+template <typename T>
+void resident_destroy(ResidentCsrOf<T> *A) {
   if (!A) return;
   lapis_hip_csr_plan_destroy(A->plan);
   if (A->pos) (void)hipFree(A->pos);
   if (A->crd) (void)hipFree(A->crd);
   if (A->val) (void)hipFree(A->val);
+}
+}  // namespace
+
+extern "C" lapis_dualview_f64 *lapis_dualview_f64_create(double *host, int64_t n) {
+  return dualview_create<lapis_dualview_f64>(host, n);
+}
+extern "C" void lapis_dualview_f64_modify_host(lapis_dualview_f64 *v) { v->modified_host = true; }
+extern "C" void lapis_dualview_f64_modify_device(lapis_dualview_f64 *v) { v->modified_device = true; }
+extern "C" void lapis_dualview_f64_sync_host(lapis_dualview_f64 *v) { dualview_sync_host<double>(v); }
+extern "C" void lapis_dualview_f64_sync_device(lapis_dualview_f64 *v) { dualview_sync_device<double>(v); }
+extern "C" void lapis_dualview_f64_destroy(lapis_dualview_f64 *v) {
+  dualview_destroy<double>(v);
+  delete v;
+}
+extern "C" lapis_dualview_f32 *lapis_dualview_f32_create(float *host, int64_t n) {
+  return dualview_create<lapis_dualview_f32>(host, n);
+}
+extern "C" void lapis_dualview_f32_modify_host(lapis_dualview_f32 *v) { v->modified_host = true; }
+extern "C" void lapis_dualview_f32_modify_device(lapis_dualview_f32 *v) { v->modified_device = true; }
+extern "C" void lapis_dualview_f32_sync_host(lapis_dualview_f32 *v) { dualview_sync_host<float>(v); }
+extern "C" void lapis_dualview_f32_sync_device(lapis_dualview_f32 *v) { dualview_sync_device<float>(v); }
+extern "C" void lapis_dualview_f32_destroy(lapis_dualview_f32 *v) {
+  dualview_destroy<float>(v);
+  delete v;
+}
+
+extern "C" lapis_resident_csr *lapis_resident_csr_create(lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd,
+                                                         lapis_memref_1d_f64 *val, const lapis_csr_specifier *spec) {
+  return resident_create<lapis_resident_csr, double>(pos, crd, val, spec);
+}
+extern "C" void lapis_resident_csr_update_values(lapis_resident_csr *A, lapis_memref_1d_f64 *val) {
+  resident_update_values<double>(A, val);
+}
+extern "C" void lapis_resident_csr_spmv(lapis_resident_csr *A, lapis_dualview_f64 *x, lapis_dualview_f64 *y) {
+  resident_spmv<double>(A, x, y);
+}
+extern "C" void lapis_resident_csr_spmm(lapis_resident_csr *A, lapis_dualview_f64 *B, int64_t k, lapis_dualview_f64 *C) {
+  resident_spmm<double>(A, B, k, C);
+}
+// func @pcg on resident operands: x (allocated by the caller, overwritten) = the solution
+extern "C" void lapis_resident_csr_pcg(lapis_resident_csr *A, lapis_dualview_f64 *b, lapis_dualview_f64 *dinv, double tol,
+                                       size_t maxiter, lapis_dualview_f64 *x, size_t *iters, double *relres) {
+  const int64_t n = A->nrows;
+  if (A->ncols != n) module_abort("pcg: A must be square");
+  if (b->n < n || x->n < n || (dinv && dinv->n < n)) module_abort("pcg: b, dinv and x need n elements");
+  if (x == b || x == dinv) module_abort("pcg: x must be a view of its own");
+  dualview_sync_device<double>(b);
+  if (dinv) dualview_sync_device<double>(dinv);
+  uint64_t it = 0;
+  double rr = 0.0;
+  check(lapis_hip_pcg_f64_i32(A->plan, n, A->pos, A->crd, A->val, b->dev, dinv ? dinv->dev : nullptr, tol, (uint64_t)maxiter,
+                              x->dev, &it, &rr, nullptr, nullptr),
+        "lapis_hip_pcg_f64_i32");
+  x->modified_device = true;
+  x->modified_host = false;
+  if (iters) *iters = (size_t)it;
+  if (relres) *relres = rr;
+}
+extern "C" void lapis_resident_csr_destroy(lapis_resident_csr *A) {
+  resident_destroy<double>(A);
+  delete A;
+}
+
+extern "C" lapis_resident_csr_f32 *lapis_resident_csr_f32_create(lapis_memref_1d_i32 *pos, lapis_memref_1d_i32 *crd,
+                                                                 lapis_memref_1d_f32 *val, const lapis_csr_specifier *spec) {
+  return resident_create<lapis_resident_csr_f32, float>(pos, crd, val, spec);
+}
+extern "C" void lapis_resident_csr_f32_update_values(lapis_resident_csr_f32 *A, lapis_memref_1d_f32 *val) {
+  resident_update_values<float>(A, val);
+}
+extern "C" void lapis_resident_csr_f32_spmv(lapis_resident_csr_f32 *A, lapis_dualview_f32 *x, lapis_dualview_f32 *y) {
+  resident_spmv<float>(A, x, y);
+}
+extern "C" void lapis_resident_csr_f32_spmm(lapis_resident_csr_f32 *A, lapis_dualview_f32 *B, int64_t k,
+                                            lapis_dualview_f32 *C) {
+  resident_spmm<float>(A, B, k, C);
+}
+extern "C" void lapis_resident_csr_f32_destroy(lapis_resident_csr_f32 *A) {
+  resident_destroy<float>(A);
   delete A;
 }
 
@@ -358,6 +462,8 @@ extern "C" void py_pcg(lapis_memref_1d_f64 **ret0, size_t *ret1, double *ret2, l
     DeviceMirror<double> dx(hx, (size_t)n, false);
     lapis_hip_csr_plan *plan = nullptr;
     check(lapis_hip_csr_plan_create(&plan, n, n, a.nnz, dpos.dev, dcrd.dev, 8, nullptr), "lapis_hip_csr_plan_create");
+    // enough iterations for the column-blocked copy to pay back where the library recommends one
+    if (maxiter >= 64) check(lapis_hip_csr_plan_analyze(plan, dcrd.dev, dval.dev, 8, nullptr), "lapis_hip_csr_plan_analyze");
     check(lapis_hip_pcg_f64_i32(plan, n, dpos.dev, dcrd.dev, dval.dev, db.dev, ddinv.dev, tol, (uint64_t)maxiter,
                                 dx.dev, &iters, &relres, nullptr, nullptr),
           "lapis_hip_pcg_f64_i32");
@@ -462,6 +568,8 @@ extern "C" void py_mht(lapis_memref_1d_f64 **ret0, lapis_memref_1d_f64 **ret1, l
     DeviceMirror<double> d1(h1, (size_t)n, false), d2(h2, (size_t)n, false);
     lapis_hip_csr_plan *plan = nullptr;
     check(lapis_hip_csr_plan_create(&plan, n, n, a.nnz, dpos.dev, dcrd.dev, 8, nullptr), "lapis_hip_csr_plan_create");
+    // two solves of up to maxiter iterations each; mht refreshes the copy's values after it has scaled the matrix
+    if (maxiter >= 32) check(lapis_hip_csr_plan_analyze(plan, dcrd.dev, dval.dev, 8, nullptr), "lapis_hip_csr_plan_analyze");
     check(lapis_hip_mht_f64_i32(plan, n, a.nnz, dpos.dev, dcrd.dev, dval.dev, dmask.dev, dd.dev, alpha, tol,
                                 (uint64_t)maxiter, d1.dev, d2.dev, nullptr),
           "lapis_hip_mht_f64_i32");

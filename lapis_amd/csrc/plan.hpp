@@ -9,6 +9,7 @@
 struct lapis_hip_csr_plan {
   lapis_hip_csr_stats stats;
   const int32_t *pos;
+  const int32_t *crd;  // the coordinates the statistics were read from (null when the plan was made without them)
   int nchunks;
   int chunk;            // non-zeros per wavefront of the row-split kernel (512, 1024 or 2048)
   int waves_per_block;  // wavefronts per workgroup of the row-split kernel

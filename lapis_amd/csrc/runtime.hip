@@ -154,6 +154,7 @@ extern "C" const char *lapis_hip_status_name(int status) {
     case LAPIS_HIP_ERR_BAD_CSR: return "LAPIS_HIP_ERR_BAD_CSR";
     case LAPIS_HIP_ERR_UNSUPPORTED_DEVICE: return "LAPIS_HIP_ERR_UNSUPPORTED_DEVICE";
     case LAPIS_HIP_ERR_PLAN_MISMATCH: return "LAPIS_HIP_ERR_PLAN_MISMATCH";
+    case LAPIS_HIP_ERR_NO_TILING: return "LAPIS_HIP_ERR_NO_TILING";
     default: return "LAPIS_HIP_ERR_UNKNOWN";
   }
 }

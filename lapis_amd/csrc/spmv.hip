@@ -718,6 +718,7 @@ extern "C" int lapis_hip_csr_plan_create(lapis_hip_csr_plan **out, int64_t nrows
   s.reference_hint = reference_hint(nrows, ends[0], ends[1]);
   s.reference_vector_length = reference_vector_length(s.reference_hint);
   p->pos = pos;
+  p->crd = crd;
   // Non-temporal loads of the streamed arrays pay when x does not fit L2 anyway (they
   // keep the stream from evicting what little of x is cached); when the gathers of a
   // chunk stay inside a window L2 can hold, plain loads are 10-15 % faster.
@@ -762,6 +763,13 @@ extern "C" int lapis_hip_csr_plan_create(lapis_hip_csr_plan **out, int64_t nrows
   }
   *out = p;
   return LAPIS_HIP_OK;
+}
+
+extern "C" int lapis_hip_csr_plan_matches(const lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, int64_t nnz,
+                                          const int32_t *pos, const int32_t *crd) {
+  if (!plan) return 0;
+  const lapis_hip_csr_stats &s = plan->stats;
+  return (s.nrows == nrows && s.ncols == ncols && s.nnz == nnz && plan->pos == pos && plan->crd == crd) ? 1 : 0;
 }
 
 extern "C" int lapis_hip_csr_plan_set_kernel(lapis_hip_csr_plan *plan, int kernel, int width) {

@@ -69,6 +69,8 @@ _SIGNATURES = {
     "lapis_hip_csr_plan_analyze": [_vp, _vp, _vp, _int, _vp],
     "lapis_hip_csr_plan_update_values": [_vp, _vp, _int, _vp],
     "lapis_hip_csr_plan_check": [_vp, _vp],
+    "lapis_hip_csr_plan_matches": [_vp, _i64, _i64, _i64, _vp, _vp],
+    "lapis_hip_csr_plan_analyze_reproducible": [_vp, _vp, _vp, _int, _vp],
     "lapis_hip_spmv_csr_f64_i32": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp],
     "lapis_hip_spmv_csr_f32_i32": [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp],
     "lapis_hip_spmm_csr_f32_i32": [_i64, _i64, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp],
@@ -79,6 +81,10 @@ _SIGNATURES = {
     "lapis_hip_dot_f64": [_i64, _vp, _vp, _dbl, _vp, _vp],
     "lapis_hip_dot_f32": [_i64, _vp, _vp, _flt, _vp, _vp],
     "lapis_hip_dot_f64_noalloc": [_i64, _vp, _vp, _dbl, _vp, _vp],
+    "lapis_hip_dot_f64_host": [_i64, _vp, _vp, _dbl, ctypes.POINTER(_dbl), _vp],
+    "lapis_hip_dot_f32_host": [_i64, _vp, _vp, _flt, ctypes.POINTER(_flt), _vp],
+    "lapis_hip_axpby_dot_f64": [_i64, _dbl, _vp, _dbl, _vp, _vp, _vp, _dbl, _vp, _vp],
+    "lapis_hip_axpby_dot_f32": [_i64, _flt, _vp, _flt, _vp, _vp, _vp, _flt, _vp, _vp],
     "lapis_hip_axpby_f64": [_i64, _dbl, _vp, _dbl, _vp, _vp, _vp],
     "lapis_hip_axpby_f32": [_i64, _flt, _vp, _flt, _vp, _vp, _vp],
     "lapis_hip_mult_f64": [_i64, _vp, _vp, _vp, _vp],
@@ -218,6 +224,16 @@ class CsrPlan:
                                                    _stream(stream)))
         return self
 
+    def analyze_reproducible(self, crd, val, stream=None):
+        """analyze() for callers that need the same bits from every run (per-wavefront layout where the copy pays)."""
+        check(self._lib.lapis_hip_csr_plan_analyze_reproducible(self._handle, _ptr(crd), _ptr(val), val.element_size(),
+                                                                _stream(stream)))
+        return self
+
+    def matches(self, nrows, ncols, nnz, pos, crd):
+        """Was this plan made for exactly this structure (sizes, number of non-zeros, position and coordinate buffers)?"""
+        return bool(self._lib.lapis_hip_csr_plan_matches(self._handle, nrows, ncols, nnz, _ptr(pos), _ptr(crd)))
+
     def update_values(self, val, stream=None):
         """Refresh the values of the column-blocked copy after ``val`` changed (no-op without a copy)."""
         check(self._lib.lapis_hip_csr_plan_update_values(self._handle, _ptr(val), val.element_size(), _stream(stream)))
@@ -312,6 +328,24 @@ def calibrate_mix(mode, x, window_bytes, stream_buf, stream_bytes, gathers, cu_c
              int(gathers), _ptr(cu_count) if cu_count is not None else None, _ptr(sink), ctypes.byref(ms),
              ctypes.byref(done), ctypes.byref(sbytes), ctypes.byref(both), _stream(stream)))
     return {"ms": ms.value, "gathers": done.value, "stream_bytes": sbytes.value, "cus_with_both_roles": both.value}
+
+
+def dot_host(x, y, init_value=0.0, stream=None):
+    """init + x . y as a Python float: the entry point that returns the scalar to the host (blocking)."""
+    lib = init()
+    out = (_dbl if x.element_size() == 8 else _flt)(0.0)
+    fn = getattr(lib, "lapis_hip_dot_%s_host" % _suffix(x))
+    check(fn(int(x.shape[0]), _ptr(x), _ptr(y), init_value, ctypes.byref(out), _stream(stream)))
+    return out.value
+
+
+def axpby_dot(a, x, b, y, dst, z, result, init_value=0.0, stream=None):
+    """dst = a*x + b*y and result = init + dst . z (z None: dst . dst) in one pass."""
+    lib = init()
+    fn = getattr(lib, "lapis_hip_axpby_dot_%s" % _suffix(x))
+    check(fn(int(x.shape[0]), a, _ptr(x), b, _ptr(y), _ptr(dst), _ptr(z) if z is not None else None, init_value,
+             _ptr(result), _stream(stream)))
+    return result
 
 
 def dot_noalloc(x, y, result, init_value=0.0, stream=None):

@@ -26,6 +26,7 @@ The pass rewrites IR; this file only DECIDES, and reports the decision as a tree
 """
 import re
 
+from . import elementwise as _ew
 from . import mlir_text as _mt
 
 HOST, DEVICE, TEAM_HANDLE = 0, 1, 2                       # executionSpace attribute values
@@ -104,6 +105,9 @@ class NestMapping:
         self.space, self.depth, self.tree = space, depth, tree
         self.vector_length_hint, self.team_size_hint = vector_length_hint, team_size_hint
         self.csr_spmv = None   # {"y", "pos", "crd", "val", "x", "elem"} when the nest is the CSR SpMV nest
+        self.depth1 = None     # match_depth1: a dot or an elementwise loop the kernel library has an entry for
+        self.csr_spmm = None   # match_csr_spmm: the CSR x dense SpMM nest
+        self.stmt = None       # the scf.parallel statement of the nest
 
     def summary(self):
         return self.tree.summary()
@@ -275,6 +279,172 @@ class _Mapper:
             return None
         return {"y": y0[0], "pos": pos, "crd": xc[1], "val": vload[0], "x": xc[0], "elem": elem}
 
+
+    # -- depth-1 nests the kernel library runs: dot, axpby / mult / scale / copy / fill --------------
+    def _load_at(self, name, iv):
+        """Memref of a one-dimensional `memref.load <m>[<iv>]` that defines `name` (casts followed), else None."""
+        name = self._follow_cast(name)
+        if name not in self.defs or self.defs[name][0].op != "memref.load":
+            return None
+        m = re.match(r"\s*(%[\w.$-]+)\s*\[\s*(%[\w.$-]+)\s*\]", self.defs[name][0].head)
+        if not m or self._follow_cast(m.group(2)) != iv:
+            return None
+        return m.group(1)
+
+    def match_depth1(self, top):
+        """What a one-level `scf.parallel` over one induction variable computes, if it is a loop the library
+        has an entry point for (the loops DenseLinalgToParallelLoops.cpp:227-272,349-393 of the reference
+        makes of linalg.dot, linalg.fill, linalg.copy and parallel linalg.generic), else None:
+
+        {"kind": "dot", "x", "y", "init", "result", "elem", "n"}  or
+        {"kind": "axpby" | "scale" | "mult" | "copy" | "fill", "dst", "arrays", "call", "elem", "n"}
+        with `call` the classification of lapis_amd/elementwise.py over `arrays`."""
+        if len(top.ivs) != 1 or top.levels != 1 or top.inner:
+            return None
+        iv, n = top.ivs[0], top.upper[0]
+        arrays = []
+
+        def element_of(name):
+            m = self._load_at(name, iv)
+            if m is None:
+                return None
+            if m not in arrays:
+                arrays.append(m)
+            return arrays.index(m)
+
+        body = [s for s in top.body if s.op not in ("scf.yield",)]
+        loads = [s for s in body if s.op == "memref.load"]
+        for s in loads:  # every load is an element at the loop index
+            mm = re.match(r"\s*(%[\w.$-]+)\s*\[\s*(%[\w.$-]+)\s*\]", s.head)
+            if not mm or self._follow_cast(mm.group(2)) != iv:
+                return None
+        arith = [s for s in body if s.op.startswith("arith.")]
+        stores = [s for s in body if s.op == "memref.store"]
+        reduces = [s for s in body if s.op == "scf.reduce"]
+        if len(loads) + len(arith) + len(stores) + len(reduces) != len(body):
+            return None
+        try:
+            if top.results == 1:  # a reduction: init + sum x[i] * y[i]
+                m = re.search(r"init\s*\(\s*(%[\w.$-]+)\s*\)\s*->\s*(\w+)", top.stmt.head)
+                if not m or stores or len(reduces) != 1 or len(reduces[0].regions) != 1 or m.group(2) not in ("f64", "f32"):
+                    return None
+                bargs, comb = reduces[0].regions[0]
+                if len(comb) != 2 or comb[0].op != "arith.addf" or sorted(self._operands(comb[0])) != sorted(bargs):
+                    return None
+                reduced = _mt._VALUE.search(reduces[0].head).group(0)
+                poly = _ew.polynomial(arith, element_of, reduced)
+                terms = {k: c for k, c in poly.terms.items() if c != ("const", 0.0)}
+                if len(terms) != 1:
+                    return None
+                (mono, coeff), = terms.items()
+                if len(mono) != 2 or coeff != ("const", 1.0):
+                    return None
+                return {"kind": "dot", "x": arrays[mono[0]], "y": arrays[mono[1]], "init": m.group(1),
+                        "result": top.stmt.results[0], "elem": m.group(2), "n": n}
+            if top.results or len(stores) != 1 or any(r.regions for r in reduces):
+                return None
+            m = re.match(r"\s*(%[\w.$-]+)\s*,\s*(%[\w.$-]+)\s*\[\s*(%[\w.$-]+)\s*\]\s*:\s*memref<\?x(\w+)>", stores[0].head)
+            if not m or self._follow_cast(m.group(3)) != iv or m.group(4) not in ("f64", "f32"):
+                return None
+            call = _ew.classify(_ew.polynomial(arith, element_of, m.group(1)))
+        except _ew.Unsupported:
+            return None
+        # coefficients have to be loop invariant: defined outside the nest
+        for expr in [c for c in call[1:] if isinstance(c, tuple)]:
+            for nm in _ew.scalar_names(expr):
+                if nm in self.defs and self._inside(self.defs[nm][0], top):
+                    return None
+        return {"kind": call[0], "dst": m.group(2), "arrays": list(arrays), "call": call, "elem": m.group(4), "n": n}
+
+    # -- the CSR x dense SpMM nest ------------------------------------------------------------------
+    def match_csr_spmm(self, top):
+        """Buffers of `C[i,j] += sum_kk val[kk] * B[crd[kk], j]`, kk in [pos[i], pos[i+1]), when `top` is that
+        nest with the rows parallel, the compressed loop sequential (`scf.for`) and the dense column loop
+        either kind -- what the sparsifier leaves for CSR x dense matmul (examples/spmm_dcsr_opdsl.py:73-110)
+        under the strategies that do not parallelise the reduction (Pipelines/Passes.h:41-56) -- else None:
+        {"C", "pos", "crd", "val", "B", "elem", "rows", "k"}."""
+        if len(top.ivs) != 1 or top.results:
+            return None
+        i = top.ivs[0]
+        fors = [s for s in top.body if s.op == "scf.for"]
+        if len(fors) != 1 or any(s.op not in ("memref.load", "arith.addi", "scf.for", "scf.reduce", "scf.yield") + _CASTS
+                                 for s in top.body):
+            return None
+        outer = fors[0]
+        m = re.match(r"\s*(%[\w.$-]+)\s*=\s*(%[\w.$-]+)\s*to\s*(%[\w.$-]+)\s*step\s*(%[\w.$-]+)", outer.head)
+        if not m or not self._is_one(m.group(4)) or "iter_args" in outer.head:
+            return None
+        kk, lo, hi = m.group(1), self._follow_cast(m.group(2)), self._follow_cast(m.group(3))
+
+        def load1(v):
+            v = self._follow_cast(v)
+            if v not in self.defs or self.defs[v][0].op != "memref.load":
+                return None
+            mm = re.match(r"\s*(%[\w.$-]+)\s*\[\s*(%[\w.$-]+)\s*\]", self.defs[v][0].head)
+            return (mm.group(1), self._follow_cast(mm.group(2))) if mm else None
+
+        plo, phi = load1(lo), load1(hi)
+        if not plo or not phi or plo[0] != phi[0] or plo[1] != i:
+            return None
+        nxt = phi[1]
+        if nxt not in self.defs or self.defs[nxt][0].op != "arith.addi":
+            return None
+        a, c = self._operands(self.defs[nxt][0])
+        if not ((self._follow_cast(a) == i and self._is_one(c)) or (self._follow_cast(c) == i and self._is_one(a))):
+            return None
+        mid = outer.regions[0][1]
+        inner = [s for s in mid if s.op in ("scf.for", "scf.parallel")]
+        if len(inner) != 1 or any(s.op not in ("memref.load", "scf.for", "scf.parallel", "scf.yield") + _CASTS for s in mid):
+            return None
+        jl = inner[0]
+        if jl.op == "scf.for":
+            mj = re.match(r"\s*(%[\w.$-]+)\s*=\s*(%[\w.$-]+)\s*to\s*(%[\w.$-]+)\s*step\s*(%[\w.$-]+)", jl.head)
+            if not mj or not self._is_one(mj.group(4)) or "iter_args" in jl.head:
+                return None
+            j, kcols = mj.group(1), mj.group(3)
+        else:
+            mj = re.match(r"\s*\(\s*(%[\w.$-]+)\s*\)\s*=\s*\([^)]*\)\s*to\s*\(\s*(%[\w.$-]+)\s*\)\s*step\s*\(\s*(%[\w.$-]+)\s*\)", jl.head)
+            if not mj or not self._is_one(mj.group(3)) or jl.results:
+                return None
+            j, kcols = mj.group(1), mj.group(2)
+        jbody = jl.regions[0][1]
+        if any(s.op not in ("memref.load", "arith.mulf", "arith.addf", "memref.store", "scf.yield", "scf.reduce") + _CASTS
+               for s in jbody):
+            return None
+        stores = [s for s in jbody if s.op == "memref.store"]
+        if len(stores) != 1:
+            return None
+
+        def load2(v):
+            v = self._follow_cast(v)
+            if v not in self.defs or self.defs[v][0].op != "memref.load":
+                return None
+            mm = re.match(r"\s*(%[\w.$-]+)\s*\[\s*(%[\w.$-]+)\s*,\s*(%[\w.$-]+)\s*\]", self.defs[v][0].head)
+            return (mm.group(1), self._follow_cast(mm.group(2)), self._follow_cast(mm.group(3))) if mm else None
+
+        ms = re.match(r"\s*(%[\w.$-]+)\s*,\s*(%[\w.$-]+)\s*\[\s*(%[\w.$-]+)\s*,\s*(%[\w.$-]+)\s*\]\s*:\s*memref<\?x\?x(\w+)>",
+                      stores[0].head)
+        if not ms or self._follow_cast(ms.group(3)) != i or self._follow_cast(ms.group(4)) != j:
+            return None
+        total, C, elem = ms.group(1), ms.group(2), ms.group(5)
+        if elem not in ("f64", "f32") or total not in self.defs or self.defs[total][0].op != "arith.addf":
+            return None
+        t0, t1 = self._operands(self.defs[total][0])
+        old, prod = (t0, t1) if load2(t0) else (t1, t0)
+        lold = load2(old)
+        if not lold or lold != (C, i, j) or prod not in self.defs or self.defs[prod][0].op != "arith.mulf":
+            return None
+        p0, p1 = self._operands(self.defs[prod][0])
+        vname, bname = (p0, p1) if load1(p0) else (p1, p0)
+        lv, lb = load1(vname), load2(bname)
+        if not lv or not lb or lv[1] != kk or lb[2] != j:
+            return None
+        lc = load1(lb[1])
+        if not lc or lc[1] != kk:
+            return None
+        return {"C": C, "pos": plo[0], "crd": lc[0], "val": lv[0], "B": lb[0], "elem": elem, "rows": top.upper[0],
+                "k": kcols}
+
     # -- the tree -----------------------------------------------------------------------------------
     def map_nest(self, top, hip_kernels=False):
         offload = not _contains(top.body, _HOST_ONLY)
@@ -300,6 +470,8 @@ class _Mapper:
                 team = self._estimate(top, [l for l in all_loops if level_of.get(id(l)) == ("range", TEAM_HANDLE, TEAM_THREAD)])
         mapping = NestMapping("device" if offload else "host", depth, tree, vec, team)
         mapping.csr_spmv = self.match_csr_spmv(top) if space == DEVICE else None
+        mapping.depth1 = self.match_depth1(top) if space == DEVICE and depth == 1 else None
+        mapping.csr_spmm = self.match_csr_spmm(top) if space == DEVICE and not mapping.csr_spmv else None
         if hip_kernels and mapping.csr_spmv:
             # the kernel library takes this nest over; its plan reads the row statistics once, so no estimate
             # (and with it no host read of the positions) is left before the launch
@@ -400,13 +572,24 @@ def map_function_body(body_text, hip_kernels=False):
     """[NestMapping] for the top-level scf.parallel nests of one function body, in program order.
     `hip_kernels`: a nest that is the CSR SpMV nest goes to the kernel library and gets no estimate."""
     stmts, _ = _mt.read_region(body_text)
+    return map_statements(stmts, hip_kernels)
+
+
+def map_statements(stmts, hip_kernels=False):
+    """map_function_body for a body that is already read: `.stmt` of every NestMapping is the caller's own
+    `scf.parallel` Statement object."""
     loops = []
     _walk_loops(stmts, None, loops)
     tops = [l for l in loops if l.parent is None]
     for t in tops:
         _set_levels(t)
     mapper = _Mapper(stmts)
-    return [mapper.map_nest(t, hip_kernels) for t in tops]
+    out = []
+    for t in tops:
+        mapping = mapper.map_nest(t, hip_kernels)
+        mapping.stmt = t.stmt
+        out.append(mapping)
+    return out
 
 
 def map_module(text, hip_kernels=False):

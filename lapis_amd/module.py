@@ -31,33 +31,44 @@ def _flatten_specifier(spec):
     return flat
 
 
-class DualView:
-    """A numpy array paired with a device copy that stays allocated between calls: the role of
-    LAPIS::DualView (LAPISSupport.hpp:136-426) with its lazy modified-host / modified-device flags.
-    ``host`` is the numpy side; after writing to it call ``modify_host()``; ``sync_host()`` brings a
-    result back (and waits for the kernels that produce it)."""
+def _value_dtype(array):
+    return numpy.float32 if numpy.asarray(array).dtype == numpy.float32 else numpy.float64
 
-    def __init__(self, lib, array):
-        self._lib = lib
-        self.host = numpy.require(array, dtype=numpy.float64, requirements=['C', 'W'])
-        self._handle = ctypes.c_void_p(lib.lapis_dualview_f64_create(self.host.ctypes.data_as(ctypes.c_void_p),
-                                                                     ctypes.c_int64(self.host.shape[0])))
+
+class DualView:
+    """A numpy array (float64, or float32 if it is given as such) paired with a device copy that stays
+    allocated between calls: the role of LAPIS::DualView (LAPISSupport.hpp:136-426) with its lazy
+    modified-host / modified-device flags.  ``host`` is the numpy side; after writing to it call
+    ``modify_host()``; ``sync_host()`` brings a result back (and waits for the kernels that produce it).
+    Arrays of more than one dimension are kept row-major; ``host`` has the caller's shape."""
+
+    def __init__(self, module, array):
+        self._module = module  # keeps the library initialised for as long as the view lives
+        self._lib = module.libHandle
+        self.dtype = _value_dtype(array)
+        self._tag = "f32" if self.dtype == numpy.float32 else "f64"
+        self.host = numpy.require(array, dtype=self.dtype, requirements=['C', 'W'])
+        create = getattr(self._lib, "lapis_dualview_%s_create" % self._tag)
+        self._handle = ctypes.c_void_p(create(self.host.ctypes.data_as(ctypes.c_void_p), ctypes.c_int64(self.host.size)))
+
+    def _call(self, what):
+        getattr(self._lib, "lapis_dualview_%s_%s" % (self._tag, what))(self._handle)
 
     def modify_host(self):
-        self._lib.lapis_dualview_f64_modify_host(self._handle)
+        self._call("modify_host")
         return self
 
     def sync_host(self):
-        self._lib.lapis_dualview_f64_sync_host(self._handle)
+        self._call("sync_host")
         return self.host
 
     def sync_device(self):
-        self._lib.lapis_dualview_f64_sync_device(self._handle)
+        self._call("sync_device")
         return self
 
     def release(self):
         if self._handle:
-            self._lib.lapis_dualview_f64_destroy(self._handle)
+            self._call("destroy")
             self._handle = None
 
     def __del__(self):
@@ -69,46 +80,100 @@ class DualView:
 
 class ResidentCsr:
     """A CSR matrix uploaded once (``LAPISModule.bind_csr``): device copies, plan and, where the library
-    recommends it, the column-blocked copy are reused by every ``spmv``."""
+    recommends it, the column-blocked copy are reused by every ``spmv`` / ``spmm`` / ``pcg``.  The values
+    are float64, or float32 if they are given as such; vector operands must have the matrix's type."""
 
     def __init__(self, module, pos, crd, val, spec):
         self._module = module  # keeps the library initialised for as long as the matrix lives
         self._lib = module.libHandle
+        self.dtype = _value_dtype(val)
+        self._prefix = "lapis_resident_csr_f32_" if self.dtype == numpy.float32 else "lapis_resident_csr_"
         pos = numpy.require(pos, dtype=numpy.int32, requirements=['C'])
         crd = numpy.require(crd, dtype=numpy.int32, requirements=['C'])
-        val = numpy.require(val, dtype=numpy.float64, requirements=['C'])
+        val = numpy.require(val, dtype=self.dtype, requirements=['C'])
         flat = _flatten_specifier(spec)
         self.shape = (int(flat[0]), int(flat[1]))
-        self._handle = ctypes.c_void_p(self._lib.lapis_resident_csr_create(
+        self._handle = ctypes.c_void_p(self._fn("create")(
             ctypes.pointer(rt.get_ranked_memref_descriptor(pos)), ctypes.pointer(rt.get_ranked_memref_descriptor(crd)),
             ctypes.pointer(rt.get_ranked_memref_descriptor(val)), flat.ctypes.data_as(ctypes.c_void_p)))
 
+    def _fn(self, what):
+        return getattr(self._lib, self._prefix + what)
+
+    def _views(self, *operands):
+        """DualViews of the operands (made for the call where numpy arrays are given) and which ones are ours."""
+        views = [v if isinstance(v, DualView) else DualView(self._module, numpy.asarray(v, dtype=self.dtype)) for v in operands]
+        for v in views:
+            if v.dtype != self.dtype:
+                raise TypeError("operand is %s, the matrix holds %s" % (v.dtype.__name__, self.dtype.__name__))
+        return views
+
     def update_values(self, val):
-        val = numpy.require(val, dtype=numpy.float64, requirements=['C'])
-        self._lib.lapis_resident_csr_update_values(self._handle, ctypes.pointer(rt.get_ranked_memref_descriptor(val)))
+        val = numpy.require(val, dtype=self.dtype, requirements=['C'])
+        self._fn("update_values")(self._handle, ctypes.pointer(rt.get_ranked_memref_descriptor(val)))
+
+    def _finish(self, out_view, given, views, operands):
+        """In-place contract for numpy operands: fetch the result, write it through to the caller's array."""
+        out = out_view.sync_host()
+        if isinstance(given, numpy.ndarray) and out is not given:
+            given[...] = out.reshape(given.shape)  # numpy.require had to copy (dtype or layout)
+            out = given
+        for v, g in zip(views, operands):
+            if v is not g:
+                v.release()
+        return out
 
     def spmv(self, x, y):
         """y += A x.  With ``DualView`` operands nothing crosses PCIe and the call returns before the kernel
         has run (``y.sync_host()`` fetches the result); numpy operands are copied in and out as
         ``LAPISModule.spmv`` does, and the updated ``y`` is returned."""
-        if isinstance(x, DualView) and isinstance(y, DualView):
-            self._lib.lapis_resident_csr_spmv(self._handle, x._handle, y._handle)
+        xv, yv = self._views(x, y)
+        self._fn("spmv")(self._handle, xv._handle, yv._handle)
+        if xv is x and yv is y:
             return y
-        xv = x if isinstance(x, DualView) else DualView(self._lib, x)
-        yv = y if isinstance(y, DualView) else DualView(self._lib, y)
-        self._lib.lapis_resident_csr_spmv(self._handle, xv._handle, yv._handle)
-        out = yv.sync_host()
-        if out is not y and isinstance(y, numpy.ndarray):
-            y[...] = out  # numpy.require had to copy (dtype or layout): keep the in-place contract
-            out = y
-        for v, given in ((xv, x), (yv, y)):
-            if v is not given:
-                v.release()
-        return out
+        return self._finish(yv, y, (xv, yv), (x, y))
+
+    def spmm(self, B, C):
+        """C += A B for row-major B (columns x k) and C (rows x k); operands as in ``spmv``."""
+        Bv, Cv = self._views(B, C)
+        if Bv.host.ndim != 2 or Cv.host.ndim != 2 or Bv.host.shape[1] != Cv.host.shape[1]:
+            raise ValueError("spmm takes two-dimensional B and C with the same number of columns")
+        if Bv.host.shape[0] < self.shape[1] or Cv.host.shape[0] < self.shape[0]:
+            raise ValueError("spmm: B needs %d rows and C %d" % (self.shape[1], self.shape[0]))
+        self._fn("spmm")(self._handle, Bv._handle, ctypes.c_int64(Bv.host.shape[1]), Cv._handle)
+        if Bv is B and Cv is C:
+            return C
+        return self._finish(Cv, C, (Bv, Cv), (B, C))
+
+    def pcg(self, b, dinv, tol, maxiter, x=None):
+        """``func @pcg`` of examples/pcg_solve.py:52 on the resident matrix (float64): returns (x, iterations,
+        relative residual).  ``dinv`` None runs unpreconditioned CG.  With a ``DualView`` x the solution stays on
+        the device (``x.sync_host()`` fetches it)."""
+        if self.dtype != numpy.float64:
+            raise TypeError("pcg is implemented for float64 matrices")
+        n = self.shape[0]
+        given_x = x
+        if x is None:
+            x = numpy.zeros(n, dtype=numpy.float64)
+        operands = [b, x] + ([dinv] if dinv is not None else [])
+        views = self._views(*operands)
+        bv, xv = views[0], views[1]
+        dv = views[2]._handle if dinv is not None else None
+        iters, relres = ctypes.c_size_t(0), ctypes.c_double(0.0)
+        self._lib.lapis_resident_csr_pcg(self._handle, bv._handle, dv, ctypes.c_double(tol), ctypes.c_size_t(maxiter),
+                                         xv._handle, ctypes.byref(iters), ctypes.byref(relres))
+        if isinstance(given_x, DualView):
+            out = given_x
+            for v, g in zip(views, operands):
+                if v is not g:
+                    v.release()
+        else:
+            out = self._finish(xv, x, views, operands)
+        return out, iters.value, relres.value
 
     def release(self):
         if self._handle:
-            self._lib.lapis_resident_csr_destroy(self._handle)
+            self._fn("destroy")(self._handle)
             self._handle = None
 
     def __del__(self):
@@ -127,18 +192,23 @@ class LAPISModule:
         self.libHandle = ctypes.CDLL(libPath)
         self.libHandle.lapis_initialize.restype = None
         self.libHandle.lapis_finalize.restype = None
-        self.libHandle.lapis_dualview_f64_create.restype = ctypes.c_void_p
-        self.libHandle.lapis_dualview_f64_create.argtypes = [ctypes.c_void_p, ctypes.c_int64]
-        for fn in ("modify_host", "modify_device", "sync_host", "sync_device", "destroy"):
-            f = getattr(self.libHandle, "lapis_dualview_f64_" + fn)
-            f.restype, f.argtypes = None, [ctypes.c_void_p]
-        self.libHandle.lapis_resident_csr_create.restype = ctypes.c_void_p
-        self.libHandle.lapis_resident_csr_update_values.restype = None
-        self.libHandle.lapis_resident_csr_update_values.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
-        self.libHandle.lapis_resident_csr_spmv.restype = None
-        self.libHandle.lapis_resident_csr_spmv.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
-        self.libHandle.lapis_resident_csr_destroy.restype = None
-        self.libHandle.lapis_resident_csr_destroy.argtypes = [ctypes.c_void_p]
+        vp = ctypes.c_void_p
+        for tag in ("f64", "f32"):
+            create = getattr(self.libHandle, "lapis_dualview_%s_create" % tag)
+            create.restype, create.argtypes = vp, [vp, ctypes.c_int64]
+            for fn in ("modify_host", "modify_device", "sync_host", "sync_device", "destroy"):
+                f = getattr(self.libHandle, "lapis_dualview_%s_%s" % (tag, fn))
+                f.restype, f.argtypes = None, [vp]
+        for prefix in ("lapis_resident_csr_", "lapis_resident_csr_f32_"):
+            fn = lambda what: getattr(self.libHandle, prefix + what)
+            fn("create").restype = vp
+            fn("update_values").restype, fn("update_values").argtypes = None, [vp, vp]
+            fn("spmv").restype, fn("spmv").argtypes = None, [vp, vp, vp]
+            fn("spmm").restype, fn("spmm").argtypes = None, [vp, vp, ctypes.c_int64, vp]
+            fn("destroy").restype, fn("destroy").argtypes = None, [vp]
+        self.libHandle.lapis_resident_csr_pcg.restype = None
+        self.libHandle.lapis_resident_csr_pcg.argtypes = [vp, vp, vp, ctypes.c_double, ctypes.c_size_t, vp,
+                                                          ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_double)]
         self.libHandle.lapis_initialize()
 
     def __del__(self):
@@ -153,8 +223,8 @@ class LAPISModule:
         return ResidentCsr(self, param0, param1, param2, param3)
 
     def dual_view(self, array):
-        """A float64 vector that keeps a device copy between calls (see ``DualView``)."""
-        return DualView(self.libHandle, array)
+        """An array (float64, or float32 if given as such) that keeps a device copy between calls (see ``DualView``)."""
+        return DualView(self, array)
 
     # func @spmv(A, x, y) -> y          (examples/spmv_noalloc.py:9, benchmarks/spmv/spmv.mlir)
     def spmv(self, param0, param1, param2, param3, param4, param5):

@@ -47,8 +47,8 @@ def test_calls_before_init_report_not_initialized():
 
 def test_status_names_are_distinct():
     lib = hip.load()
-    names = {lib.lapis_hip_status_name(i) for i in range(7)}
-    assert len(names) == 7 and lib.lapis_hip_status_name(99) == b"LAPIS_HIP_ERR_UNKNOWN"
+    names = {lib.lapis_hip_status_name(i) for i in range(8)}
+    assert len(names) == 8 and lib.lapis_hip_status_name(99) == b"LAPIS_HIP_ERR_UNKNOWN"
 
 
 def test_stats_struct_matches_header_layout():

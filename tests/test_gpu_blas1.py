@@ -86,3 +86,52 @@ def test_many_dots_in_flight_use_separate_scratch(gpu):
     torch.cuda.synchronize()
     want = [float((x.cpu().numpy() ** 2).sum()) for x in xs]
     assert np.allclose(res.cpu().numpy(), want, rtol=1e-13)
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+@pytest.mark.parametrize("n", [0, 1, 3, 1000, 4097, 1 << 20, (1 << 20) + 3])
+def test_dot_with_its_result_on_the_host(gpu, oracle, dtype, n):
+    # the entry emitted code calls where the reference reduces into a host scalar: same bits as the
+    # device-scalar entry, and the oracle's value within the reordering tolerance
+    x, y = gen.uniform_vector(n, 21, dtype=dtype), gen.uniform_vector(n, 22, dtype=dtype)
+    dx, dy = dev(x), dev(y)
+    got = gpu.dot_host(dx, dy, 0.5)
+    res = torch.zeros(1, dtype=dx.dtype, device="cuda")
+    gpu.dot(dx, dy, res, 0.5)
+    torch.cuda.synchronize()
+    assert np.asarray(got, dtype=dtype) == res.cpu().numpy()[0]
+    want = oracle.dot(x.astype(np.float64), y.astype(np.float64), 0.5)
+    scale = float(np.abs(x.astype(np.float64) * y.astype(np.float64)).sum()) + 0.5
+    assert abs(got - want) <= (1e-12 if dtype == np.float64 else 1e-5) * scale
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+@pytest.mark.parametrize("n", [1, 2, 255, 4096, 100003, 1 << 21])
+@pytest.mark.parametrize("other_z", [False, True])
+def test_fused_axpby_dot_has_the_bits_of_the_two_calls(gpu, dtype, n, other_z):
+    # r = r - alpha * Ap followed by r . r (examples/pcg_solve.py:80-82) in one pass
+    x, y, z = (gen.uniform_vector(n, s, dtype=dtype) for s in (31, 32, 33))
+    a, b = 1.0, -0.37
+    dx, dy, dz = dev(x), dev(y), dev(z)
+    dst1, res1 = torch.empty_like(dx), torch.zeros(1, dtype=dx.dtype, device="cuda")
+    gpu.axpby(a, dx, b, dy, dst1)
+    gpu.dot(dst1, dz if other_z else dst1, res1, 0.25)
+    dst2, res2 = dx.clone(), torch.zeros(1, dtype=dx.dtype, device="cuda")  # in place on x, as CG does with r
+    gpu.axpby_dot(a, dst2, b, dy, dst2, dz if other_z else None, res2, 0.25)
+    torch.cuda.synchronize()
+    assert torch.equal(dst1, dst2)
+    assert torch.equal(res1, res2)
+    want = dtype(a) * x + dtype(b) * y  # separate multiply and add, as the oracle's axpby
+    assert np.array_equal(dst2.cpu().numpy(), want.astype(dtype))
+
+
+def test_fused_axpby_dot_on_unaligned_buffers_stays_within_tolerance(gpu):
+    n = 5001
+    x, y = gen.uniform_vector(n + 1, 41), gen.uniform_vector(n + 1, 42)
+    dx, dy = dev(x)[1:], dev(y)[1:]  # 8 bytes past a 16-byte boundary
+    dst, res = torch.empty(n, dtype=torch.float64, device="cuda"), torch.zeros(1, dtype=torch.float64, device="cuda")
+    gpu.axpby_dot(2.0, dx, -1.0, dy, dst, None, res)
+    torch.cuda.synchronize()
+    want = 2.0 * x[1:] + -1.0 * y[1:]
+    assert np.array_equal(dst.cpu().numpy(), want)
+    assert abs(res.item() - float(want @ want)) <= 1e-12 * float(want @ want)

@@ -193,3 +193,50 @@ def test_cg_without_a_plan_builds_the_copy_when_it_can_pay_back(gpu, oracle):
         ig, rg = gpu.pcg(None, n, dev(pos), dev(crd), dev(val), dev(b), None, 1e-10, maxiter, x)
         xo, io, ro = oracle.pcg(pos, crd, val, b, np.ones(n), 1e-10, maxiter)
         assert abs(ig - io) <= 1 and np.allclose(x.cpu().numpy(), xo, rtol=1e-7, atol=1e-9)
+
+
+def _arrow_spd(n, long_len, seed):
+    """SPD matrix without empty rows whose first row (and column) has `long_len` entries: symmetric,
+    strictly diagonally dominant with a unit diagonal, the other rows a tridiagonal band plus their entry in
+    the long column."""
+    import scipy.sparse as sp
+    rng = np.random.Generator(np.random.PCG64(seed))
+    cols = np.sort(rng.choice(np.arange(2, n), size=long_len - 2, replace=False))
+    w = -rng.random(cols.shape[0]) * 0.5 - 0.1
+    arrow = sp.coo_matrix((w, (np.zeros_like(cols), cols)), shape=(n, n))
+    band = sp.diags([-np.ones(n - 1)], [1], shape=(n, n))
+    off = sp.csr_matrix(arrow + band)
+    off = off + off.T
+    diag = np.asarray(abs(off).sum(axis=1)).ravel() + 1.0
+    # scaled to a unit diagonal: the long row would otherwise give CG a condition number in the thousands,
+    # and ten iterations would amplify rounding differences of the dot products to 1e-7
+    scale = sp.diags(1.0 / np.sqrt(diag))
+    A = sp.csr_matrix(scale @ (off + sp.diags(diag)) @ scale)
+    A.sort_indices()
+    return A
+
+
+@pytest.mark.parametrize("chunk,waves", [(512, 8), (512, 4), (1024, 2), (2048, 4)])
+@pytest.mark.parametrize("n,long_len", [(20011, 9000), (4099, 3000), (70001, 40000)])
+def test_cg_on_the_row_split_kernel_with_rows_cut_by_many_chunks(gpu, oracle, monkeypatch, chunk, waves, n, long_len):
+    # The CG driver completes the rows the row-split kernel cuts at chunk boundaries inside its p.Ap kernel.
+    # A first row of thousands of entries is cut by 16 and more boundaries (the whole-wavefront branch), odd n
+    # exercises the vector tail, a small matrix has fewer chunks than the p.Ap grid has blocks.
+    monkeypatch.setenv("LAPIS_HIP_SPMV_CHUNK", str(chunk))
+    monkeypatch.setenv("LAPIS_HIP_SPMV_WAVES", str(waves))
+    A = _arrow_spd(n, long_len, 7 + n)
+    pos, crd, val = A.indptr.astype(np.int32), A.indices.astype(np.int32), A.data.astype(np.float64)
+    assert (np.diff(pos) > 0).all() and np.diff(pos).max() >= long_len
+    b = gen.uniform_vector(n, 5, dtype=np.float64)
+    for dinv in (None, 1.0 / A.diagonal()):
+        xo, io, ro = oracle.pcg(pos, crd, val, b, dinv if dinv is not None else np.ones(n), 0.0, 10)
+        dpos, dcrd = dev(pos), dev(crd)
+        plan = gpu.CsrPlan(n, n, dpos, dcrd)
+        plan.set_kernel(3)  # NNZSPLIT whatever the statistics say
+        assert plan.stats()["kernel_name"] == "nnzsplit" and plan.stats()["chunk"] == chunk
+        x = torch.full((n,), 3.0, dtype=torch.float64, device="cuda")
+        iters, relres = gpu.pcg(plan, n, dpos, dcrd, dev(val), dev(b), dev(dinv) if dinv is not None else None, 0.0, 10, x)
+        assert iters == io == 10
+        assert np.allclose(x.cpu().numpy(), xo, rtol=1e-9, atol=1e-12)
+        assert abs(relres - ro) <= 1e-7 * ro
+        plan.destroy()

@@ -309,3 +309,77 @@ def test_resident_matrix_gets_the_column_blocked_copy_where_recommended(gpu, ora
     y2 = np.zeros(A.nrows)
     Ad.spmv(x, y2)
     assert np.all(np.abs(y2 - 0.5 * want) <= 1e-12 * np.maximum(scale, 1e-300))
+
+
+def test_resident_fp32_matrix_spmv_and_spmm(gpu, oracle):
+    # LAPIS::DualView is a template over the element type (LAPISSupport.hpp:136): resident operands exist
+    # for float as for double, and for the SpMM of examples/spmm_dcsr_opdsl.py:73-110 as for SpMV
+    from lapis_amd.module import LAPISModule
+    mod = LAPISModule()
+    A = gen.poisson_random(30000, 11.0, seed=71)
+    A = gen.CSR(A.nrows, A.ncols, A.pos, A.crd, A.val.astype(np.float32))
+    spec = ((A.nrows, A.ncols), (A.nrows + 1, A.nnz, A.nnz))
+    Ad = mod.bind_csr(A.pos, A.crd, A.val, spec)
+    assert Ad.dtype == np.float32
+    x = gen.uniform_vector(A.ncols, 72, dtype=np.float32)
+    want = np.zeros(A.nrows, np.float32)
+    oracle.spmv(A.pos, A.crd, A.val, x, want)
+    scale = oracle.spmv_abs_scale(A.pos, A.crd, A.val, x)
+    y = np.zeros(A.nrows, np.float32)
+    assert Ad.spmv(x, y) is y
+    assert np.all(np.abs(y.astype(np.float64) - want) <= 1e-5 * np.maximum(scale, 1e-30))
+    xv, yv = mod.dual_view(x.copy()), mod.dual_view(np.zeros(A.nrows, np.float32))
+    assert xv.dtype == np.float32
+    Ad.spmv(xv, yv)
+    assert np.all(yv.host == 0.0)
+    assert np.all(np.abs(yv.sync_host().astype(np.float64) - want) <= 1e-5 * np.maximum(scale, 1e-30))
+    with pytest.raises(TypeError):
+        Ad.spmv(mod.dual_view(np.zeros(A.ncols)), yv)  # a float64 view against a float32 matrix
+    for k in (1, 7, 64):
+        B = gen.uniform_matrix(A.ncols, k, 73).astype(np.float32)
+        C0 = gen.uniform_matrix(A.nrows, k, 74).astype(np.float32)
+        Cw = C0.copy()
+        oracle.spmm(A.pos, A.crd, A.val, B, Cw)
+        C = C0.copy()
+        assert Ad.spmm(B, C) is C
+        assert np.allclose(C, Cw, rtol=2e-5, atol=2e-5 * 11 * 1.0)
+        Bv, Cv = mod.dual_view(B.copy()), mod.dual_view(C0.copy())
+        Ad.spmm(Bv, Cv)
+        assert np.array_equal(Cv.host, C0)  # stale until asked for
+        assert np.allclose(Cv.sync_host(), Cw, rtol=2e-5, atol=2e-5 * 11 * 1.0)
+    Ad.release()
+
+
+def test_resident_pcg_and_the_module_entry_reach_the_column_blocked_kernel(gpu):
+    # a symmetric, strictly diagonally dominant matrix with uniformly random columns and more than 2^20
+    # non-zeros: the library recommends the column-blocked copy; with maxiter >= 64 py_pcg asks for it
+    import scipy.sparse as sp
+    import scipy.sparse.linalg as spla
+    from lapis_amd.module import LAPISModule
+    R = gen.poisson_random(400000, 2.0, seed=81)
+    R = sp.csr_matrix((R.val, R.crd, R.pos), shape=(R.nrows, R.ncols))
+    S = R + R.T
+    S = S + sp.diags(np.asarray(abs(S).sum(axis=1)).ravel() + 1.0)
+    S = sp.csr_matrix(S)
+    S.sort_indices()
+    n = S.shape[0]
+    pos, crd, val = S.indptr.astype(np.int32), S.indices.astype(np.int32), S.data.astype(np.float64)
+    assert val.shape[0] > (1 << 20)
+    xs = gen.uniform_vector(n, 82)
+    b = S @ xs
+    dinv = 1.0 / S.diagonal()
+    spec = ((n, n), (n + 1, val.shape[0], val.shape[0]))
+    mod = LAPISModule()
+    x1, it1, rr1 = mod.pcg(pos, crd, val, spec, b, dinv, 1e-10, 100)   # analysed: maxiter >= 64
+    x2, it2, rr2 = mod.pcg(pos, crd, val, spec, b, dinv, 1e-10, 63)    # not analysed: plain CSR kernel
+    assert rr1 <= 1e-10 and rr2 <= 1e-10 and abs(int(it1) - int(it2)) <= 1
+    assert np.allclose(x1, xs, rtol=1e-7, atol=1e-9) and np.allclose(x2, xs, rtol=1e-7, atol=1e-9)
+    Ad = mod.bind_csr(pos, crd, val, spec)
+    x3, it3, rr3 = Ad.pcg(b, dinv, 1e-10, 100)
+    assert rr3 <= 1e-10 and abs(int(it3) - int(it1)) <= 1 and np.allclose(x3, xs, rtol=1e-7, atol=1e-9)
+    xv = mod.dual_view(np.zeros(n))
+    out, it4, rr4 = Ad.pcg(mod.dual_view(b.copy()), None, 1e-10, 200, x=xv)   # unpreconditioned, result left on the device
+    assert out is xv and rr4 <= 1e-10
+    assert np.allclose(xv.sync_host(), xs, rtol=1e-7, atol=1e-9)
+    assert np.linalg.norm(S @ xv.host - b) <= 2e-10 * np.linalg.norm(b)
+    Ad.release()

@@ -205,7 +205,7 @@ def test_column_blocked_copy_refuses_what_it_cannot_encode(gpu):
     plan = gpu.CsrPlan(1, 1 << 23, pos, crd)
     with pytest.raises(gpu.LapisHipError) as e:
         plan.build_colblock(crd, dev(np.ones(1)), layout="wave")
-    assert e.value.status_name == "LAPIS_HIP_ERR_INVALID_ARGUMENT"
+    assert e.value.status_name == "LAPIS_HIP_ERR_NO_TILING"
     with pytest.raises(gpu.LapisHipError):
         plan.set_kernel(4)  # nothing was built
 
@@ -439,6 +439,75 @@ def test_analyze_builds_the_copy_only_where_it_is_recommended(gpu, oracle):
     plan = gpu.CsrPlan(L.nrows, L.ncols, lp, lc)
     plan.analyze(lc, lv)
     assert plan.stats()["kernel_name"] == "nnzsplit" and plan.stats()["colblock_layout_name"] is None
+
+
+def test_a_kept_plan_is_never_used_on_another_structure_in_the_same_buffers(gpu, oracle):
+    # What emitted code that keeps a plan between calls of a generated function has to survive: the
+    # function's operands are uploaded anew at every call and a second matrix of the same shape lands at
+    # the same device addresses.  lapis_hip_csr_plan_matches tells the plan of A from matrix B (another
+    # number of non-zeros); with the plan rebuilt the answer is B's, never A's.
+    n = 20000
+    A = gen.poisson_random(n, 9.0, seed=51)
+    B = gen.poisson_random(n, 5.0, seed=52)
+    assert A.nnz > B.nnz and A.nrows == B.nrows and A.ncols == B.ncols
+    x = gen.uniform_vector(n, 53)
+    pos = torch.empty(n + 1, dtype=torch.int32, device="cuda")
+    crd = torch.empty(A.nnz, dtype=torch.int32, device="cuda")
+    val = torch.empty(A.nnz, dtype=torch.float64, device="cuda")
+    dx = dev(x)
+
+    def upload(M):
+        pos.copy_(torch.from_numpy(M.pos))
+        crd[:M.nnz].copy_(torch.from_numpy(M.crd))
+        val[:M.nnz].copy_(torch.from_numpy(M.val))
+
+    def multiply(plan, M):
+        y = torch.zeros(n, dtype=torch.float64, device="cuda")
+        gpu.spmv(plan, n, n, pos, crd, val, dx, y)
+        torch.cuda.synchronize()
+        want = np.zeros(n)
+        oracle.spmv(M.pos, M.crd, M.val, x, want)
+        return y.cpu().numpy(), want, oracle.spmv_abs_scale(M.pos, M.crd, M.val, x)
+
+    upload(A)
+    plan = gpu.CsrPlan(n, n, pos, crd, nnz=A.nnz)
+    got, want, scale = multiply(plan, A)
+    assert_rows_close(got, want, scale, np.float64, "A with its own plan")
+    assert plan.matches(n, n, A.nnz, pos, crd)
+    upload(B)  # same buffers, same shape, other structure
+    assert not plan.matches(n, n, B.nnz, pos, crd), "the plan of A must not pass for B"
+    assert not plan.matches(n, n, A.nnz, pos, dev(A.crd)) and not plan.matches(n + 1, n, A.nnz, pos, crd)
+    plan.destroy()
+    plan = gpu.CsrPlan(n, n, pos, crd, nnz=B.nnz)  # what the emitted call does on a mismatch
+    got, want, scale = multiply(plan, B)
+    assert_rows_close(got, want, scale, np.float64, "B after the rebuild")
+    wrong = np.zeros(n)
+    oracle.spmv(A.pos, A.crd, A.val, x, wrong)
+    assert not np.allclose(got, wrong)
+    plan.destroy()
+
+
+def test_reproducible_analysis_gives_the_same_bits_every_run(gpu, oracle):
+    A = gen.poisson_random(600000, 4.0, seed=31)
+    x = gen.uniform_vector(A.ncols, 32)
+    pos, crd, val, dx = dev(A.pos), dev(A.crd), dev(A.val), dev(x)
+    plan = gpu.CsrPlan(A.nrows, A.ncols, pos, crd)
+    plan.analyze_reproducible(crd, val)
+    s = plan.stats()
+    assert s["kernel_name"] == "colblock" and s["colblock_layout_name"] == "wave"
+    runs = []
+    for _ in range(3):
+        y = torch.zeros(A.nrows, dtype=torch.float64, device="cuda")
+        gpu.spmv(plan, A.nrows, A.ncols, pos, crd, val, dx, y)
+        torch.cuda.synchronize()
+        runs.append(y.cpu().numpy())
+    assert np.array_equal(runs[0], runs[1]) and np.array_equal(runs[0], runs[2])
+    want = np.zeros(A.nrows)
+    oracle.spmv(A.pos, A.crd, A.val, x, want)
+    assert_rows_close(runs[0], want, oracle.spmv_abs_scale(A.pos, A.crd, A.val, x), np.float64, "reproducible")
+    plan.analyze(crd, val)  # the other layout on request: the copy is rebuilt, not reused
+    assert plan.stats()["colblock_layout_name"] == "group"
+    plan.destroy()
 
 
 @pytest.mark.parametrize("kernel", ["nnzsplit", "rowblock"])
