@@ -268,7 +268,7 @@ def run_spmv(args, cfg):
         torch.cuda.synchronize()
         update_ms = (time.perf_counter() - t0) / 5 * 1e3
     family = "colgroup" if stats["colblock_layout_name"] == "group" else stats["kernel_name"]
-    kernel_name = "spmv_%s_kernel<%s>" % (family, "double" if dtype == np.float64 else "float")
+    kernel_name = "%s<%s>" % (plan.kernel_name(), "double" if dtype == np.float64 else "float")
     achieved = bytes_step / (kt["mean_ms"] * 1e-3) / 1e9
     out = {
         "metric": "CSR SpMV %s achieved HBM GB/s" % ("fp64" if dtype == np.float64 else "fp32"),
@@ -289,7 +289,7 @@ def run_spmv(args, cfg):
         "gflops": 2.0 * A.nnz / (ms * 1e-3) / 1e9,
         "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": traffic_from_profiles("%s_config%d" % (family, cfg), kt["mean_ms"]) if cfg else None,
+                     "traffic": traffic_from_profiles("%s_config%d" % (plan.kernel_name()[5:-7], cfg), kt["mean_ms"]) if cfg else None,
                      "traffic_source": TRAFFIC_SOURCE,
                      "kernel_ms_mean": kt["mean_ms"], "kernel_ms_median": kt["median_ms"],
                      "kernel_ms_min": kt["min_ms"], "launches_timed": kt["count"]},
@@ -490,7 +490,7 @@ def run_cg(args):
                    "final_relres": relres},
         "pct_of_hbm_peak": 100.0 * bytes_step / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "gflops": (2.0 * A.nnz + 2 * 2 * n + 3 * 3 * n) / (ms * 1e-3) / 1e9,
-        "roofline": {"bound": "hbm", "kernel": "spmv_%s_kernel<double>" % plan.stats()["kernel_name"],
+        "roofline": {"bound": "hbm", "kernel": "%s<double>" % plan.kernel_name(),
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": traffic_from_profiles("cg_spmv_config5", kt["mean_ms"]),
                      "traffic_source": TRAFFIC_SOURCE,

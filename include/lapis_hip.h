@@ -201,6 +201,11 @@ int lapis_hip_csr_plan_update_values(lapis_hip_csr_plan *plan, const void *val, 
  * pos[n] and pos[0] on the host every call (KokkosLoopMapping.cpp:290-322). */
 int lapis_hip_csr_plan_matches(const lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, int64_t nnz,
                                const int32_t *pos, const int32_t *crd);
+/* Name of the SpMV kernel a launch with `plan` runs ("spmv_subwarp_kernel", "spmv_rowblock_kernel",
+ * "spmv_nnzsplit_kernel", "spmv_colblock_kernel", "spmv_colgroup_kernel", "spmv_colgroup_pc_kernel"; ""
+ * for NULL): benchmark lines and profiles name the kernel they timed with it.  No counterpart in the
+ * reference, whose kernel is fixed when the module is compiled (KokkosLoopMapping.cpp:888-921). */
+const char *lapis_hip_csr_plan_kernel_name(const lapis_hip_csr_plan *plan);
 /* lapis_hip_csr_plan_analyze for callers that need the same bits from every run: where the
  * copy pays it is built in the per-wavefront layout (LAPIS_HIP_COLBLOCK_WAVE, wave-private
  * row sums in a fixed order) instead of the faster workgroup layout, whose LDS atomics fix

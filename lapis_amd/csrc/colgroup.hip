@@ -160,7 +160,7 @@ __global__ __launch_bounds__(THREADS) void spmv_colgroup_kernel(int nrows, int r
 // whatever it has in flight: loads of one wavefront return in issue order, so the wait
 // for a gather that hits L2 is also a wait for the entry loads issued before it, which
 // come from HBM.  Here the roles are split.  PROD wavefronts of the workgroup only
-// stream: 512 entries (index words and values, 128-bit loads) per step, two steps in
+// stream: 512 entries (index words and values, 128-bit loads) per step, one step in
 // flight, handed over through a ring of kPcSlots x 512 entries in LDS.  The other
 // wavefronts only consume: they copy a chunk from the ring into registers, give the slot
 // back, gather x and add into the row sums.  Chunk k is loaded by producer k % PROD,
@@ -217,7 +217,7 @@ __global__ __launch_bounds__(THREADS) void spmv_colgroup_pc_kernel(int nrows, in
   constexpr int NVV = kPcChunk / (64 * VPER);    // value vectors per lane and chunk (4 fp64, 2 fp32)
   constexpr int EPL = kPcChunk / 64;             // entries per consumer lane and chunk (8)
   constexpr int CONS = THREADS / 64 - PROD;
-  constexpr int DEPTH = 2;                       // chunks a producer has in flight (4 measured slower)
+  constexpr int DEPTH = 1;                       // chunks a producer has in flight
   static_assert(CONS >= 1 && PROD >= 1, "both roles need a wavefront");
   extern __shared__ __align__(16) unsigned char colgroup_lds[];
   double *acc = reinterpret_cast<double *>(colgroup_lds);
@@ -269,23 +269,17 @@ __global__ __launch_bounds__(THREADS) void spmv_colgroup_pc_kernel(int nrows, in
       pc_flag_store(ready + slot, round + 1);
       return true;
     };
-    // two register sets taken in turns, so that the loads of one chunk stay in flight while the
-    // other goes to the ring (a copy from one set to the other would wait for them)
-    // DEPTH register sets taken in turns: the loads of the others stay in flight while one goes to the
-    // ring (a copy between sets would wait for them).  The refill is unconditional (past the end it
-    // repeats the last chunk, which nobody takes): behind a condition the compiler no longer knows how
-    // many loads are in flight and waits for all of them.
+    // ONE chunk in flight per producer: wait for it, hand it over, ask for the next.  Keeping more of
+    // the copy in flight is slower here (two chunks per producer, refilled in turns: config 2 in
+    // 0.30-0.31 ms against 0.28): a streamed line waits for HBM, and while it does it holds room in the
+    // compute unit's memory pipeline that the consumers' gathers, which come back from L2, would use.
     if (wave < nchunks) {
       int k = wave;
-#pragma unroll
-      for (int d = 0; d < DEPTH; ++d) load_chunk(min(k + d * PROD, nchunks - 1), ci[d], cv[d]);
+      load_chunk(k, ci[0], cv[0]);
       while (ok && k < nchunks) {
-#pragma unroll
-        for (int d = 0; d < DEPTH; ++d) {
-          if (ok && k < nchunks) ok = hand_over(k, ci[d], cv[d]);
-          load_chunk(min(k + DEPTH * PROD, nchunks - 1), ci[d], cv[d]);
-          k += PROD;
-        }
+        ok = hand_over(k, ci[0], cv[0]);
+        k += PROD;
+        load_chunk(min(k, nchunks - 1), ci[0], cv[0]);
       }
     }
   } else {
@@ -512,6 +506,8 @@ int launch_colgroup_pc(const lapis_hip_csr_plan *p, const T *x, T *y, hipStream_
               : launch_colgroup_pc_cfg<T, THREADS, PROD, false>(p, x, y, st)
   switch (p->colblock_pc_threads * 16 + p->colblock_pc_prod) {
     LAPIS_PC_CASE(1024, 4);
+    LAPIS_PC_CASE(1024, 2);
+    LAPIS_PC_CASE(768, 2);
     LAPIS_PC_CASE(1024, 6);
     LAPIS_PC_CASE(768, 3);
     LAPIS_PC_CASE(640, 4);
@@ -749,12 +745,16 @@ int build_colgroup(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int 
   {
     // Producer and consumer wavefronts: the ring and the tile pointers have to fit beside the row sums,
     // and a consumer lane finds its slice by walking the tile pointers, which wants tiles of some size.
-    // LAPIS_HIP_COLBLOCK_PC = n > 0 selects the kernel with n producer wavefronts (1024 threads: 4 or
-    // 6; 768: 3; 640: 4; 512: 2 or 3 -- LAPIS_HIP_COLBLOCK_PC_THREADS).  It is not the default: on
-    // MI355X it runs config 2 in 0.294-0.32 ms against 0.305 ms and config 3 in 0.174-0.191 ms against
-    // 0.160 ms for the kernel whose wavefronts do both.
-    int prod = env_or("LAPIS_HIP_COLBLOCK_PC", 0);
-    const int pc_threads = env_or("LAPIS_HIP_COLBLOCK_PC_THREADS", 1024);
+    // Instantiated: 1024 threads with 2, 4 or 6 producers; 768 with 2 or 3; 640 with 4; 512 with 2 or 3.
+    // LAPIS_HIP_COLBLOCK_PC unset: chosen here; 0: never; n > 0: n producers of LAPIS_HIP_COLBLOCK_PC_THREADS.
+    int prod = env_or("LAPIS_HIP_COLBLOCK_PC", -1);
+    int pc_threads = env_or("LAPIS_HIP_COLBLOCK_PC_THREADS", 1024);
+    if (prod < 0) {
+      // doubles in request-bound tiles (the rule that also picks 512 threads) gain 8 % from the split
+      // (config 2: 0.280 against 0.306 ms); floats and dense tiles lose (config 3: 0.168-0.18 against 0.160 ms)
+      prod = (sizeof(T) == 8 && threads == 512) ? 2 : 0;
+      pc_threads = 512;
+    }
     if (colgroup_pc_lds_bytes(rows, nslices, (int)sizeof(T)) > 160 * 1024) prod = 0;
     p->colblock_pc_prod = std::max(0, prod);
     p->colblock_pc_threads = pc_threads;

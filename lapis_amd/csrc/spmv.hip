@@ -765,6 +765,19 @@ extern "C" int lapis_hip_csr_plan_create(lapis_hip_csr_plan **out, int64_t nrows
   return LAPIS_HIP_OK;
 }
 
+extern "C" const char *lapis_hip_csr_plan_kernel_name(const lapis_hip_csr_plan *plan) {
+  if (!plan) return "";
+  switch (plan->stats.kernel) {
+    case LAPIS_HIP_SPMV_SUBWARP: return "spmv_subwarp_kernel";
+    case LAPIS_HIP_SPMV_ROWBLOCK: return "spmv_rowblock_kernel";
+    case LAPIS_HIP_SPMV_NNZSPLIT: return "spmv_nnzsplit_kernel";
+    case LAPIS_HIP_SPMV_COLBLOCK:
+      if (!plan->colblock_group) return "spmv_colblock_kernel";
+      return plan->colblock_pc_prod > 0 ? "spmv_colgroup_pc_kernel" : "spmv_colgroup_kernel";
+    default: return "";
+  }
+}
+
 extern "C" int lapis_hip_csr_plan_matches(const lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, int64_t nnz,
                                           const int32_t *pos, const int32_t *crd) {
   if (!plan) return 0;

@@ -103,7 +103,8 @@ _SIGNATURES = {
 
 # every symbol include/lapis_hip.h declares
 EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + ["lapis_hip_last_error", "lapis_hip_status_name",
-                                             "lapis_hip_spmm_last_kernel", "lapis_hip_kernel_timing_median_ms"])
+                                             "lapis_hip_spmm_last_kernel", "lapis_hip_kernel_timing_median_ms",
+                                             "lapis_hip_csr_plan_kernel_name"])
 
 _lib = None
 
@@ -124,6 +125,8 @@ def load(path=None):
         fn.restype = _int
     lib.lapis_hip_last_error.restype = ctypes.c_char_p
     lib.lapis_hip_spmm_last_kernel.restype = ctypes.c_char_p
+    lib.lapis_hip_csr_plan_kernel_name.restype = ctypes.c_char_p
+    lib.lapis_hip_csr_plan_kernel_name.argtypes = [_vp]
     lib.lapis_hip_kernel_timing_median_ms.restype = _dbl
     lib.lapis_hip_kernel_timing_median_ms.argtypes = []
     lib.lapis_hip_status_name.restype = ctypes.c_char_p
@@ -229,6 +232,10 @@ class CsrPlan:
         check(self._lib.lapis_hip_csr_plan_analyze_reproducible(self._handle, _ptr(crd), _ptr(val), val.element_size(),
                                                                 _stream(stream)))
         return self
+
+    def kernel_name(self):
+        """Name of the SpMV kernel a launch with this plan runs."""
+        return self._lib.lapis_hip_csr_plan_kernel_name(self._handle).decode()
 
     def matches(self, nrows, ncols, nnz, pos, crd):
         """Was this plan made for exactly this structure (sizes, number of non-zeros, position and coordinate buffers)?"""
