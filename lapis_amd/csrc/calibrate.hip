@@ -6,11 +6,12 @@
 // gathers) and/or gathers doubles from a window of x.  The window size decides where
 // the gathers hit (16 KB: the vector cache of the CU; 1 MB: L2; 64 MB: HBM), and
 // `lanes_per_line` consecutive lanes of a wave instruction share one 128-byte line,
-// which the address unit merges into one request.  Measured on MI355X: a streamed
-// line and an L2-hit gather line each take their own time and the two ADD UP
-// (805 MB stream 0.118 ms; 67 M single-line gathers 0.246 ms; both 0.417 ms), as if
-// every CU could keep a fixed number of line requests in flight whatever they are
-// (256 lines fit the numbers: the 32 KB of its vector cache).
+// which the address unit merges into one request.  Measured on MI355X with wavefronts
+// that do both: a streamed line and an L2-hit gather line each take their own time and
+// the two ADD UP (805 MB stream 0.118 ms; 67 M single-line gathers 0.246 ms; both
+// 0.417 ms).  Wavefronts or workgroups with one role each overlap the two by about a
+// fifth (lapis_hip_calibrate_mix: 42 M gather lines + 805 MB in 0.215-0.23 ms against
+// 0.277 ms for the sum of the parts and 0.262-0.295 ms for wavefronts that do both).
 // bench.py turns the two rates into the floor of the column-blocked SpMV kernels.
 //
 // lapis_hip_calibrate_mix varies the arrangement: wavefronts per CU, loads in flight,
