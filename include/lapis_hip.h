@@ -379,13 +379,16 @@ int lapis_hip_axpby_f32(int64_t n, float a, const float *x, float b, const float
                         lapis_hip_stream_t stream);
 /* dst[i] = x[i]*y[i] (examples/pcg_solve.py:40-47). */
 int lapis_hip_mult_f64(int64_t n, const double *x, const double *y, double *dst, lapis_hip_stream_t stream);
+int lapis_hip_mult_f32(int64_t n, const float *x, const float *y, float *dst, lapis_hip_stream_t stream);
 /* dst[i] = x[i]/y[i] (linalg.div of examples/hitting_times.py:120,146). */
 int lapis_hip_div_f64(int64_t n, const double *x, const double *y, double *dst, lapis_hip_stream_t stream);
+int lapis_hip_div_f32(int64_t n, const float *x, const float *y, float *dst, lapis_hip_stream_t stream);
 /* dst[i] = v (linalg.fill, examples/pcg_solve.py:15-17). */
 int lapis_hip_fill_f64(int64_t n, double v, double *dst, lapis_hip_stream_t stream);
 int lapis_hip_fill_f32(int64_t n, float v, float *dst, lapis_hip_stream_t stream);
 /* dst[i] = src[i] (linalg.copy, examples/pcg_solve.py:65-67). */
 int lapis_hip_copy_f64(int64_t n, const double *src, double *dst, lapis_hip_stream_t stream);
+int lapis_hip_copy_f32(int64_t n, const float *src, float *dst, lapis_hip_stream_t stream);
 /* val[j] *= alpha in place (scale_csr, examples/hitting_times.py:51-71). */
 int lapis_hip_scale_f64(int64_t n, double alpha, double *val, lapis_hip_stream_t stream);
 

@@ -19,12 +19,20 @@ A module that is already lowered to loops binds too: a function whose one `scf.p
 SpMV nest the sparsifier produces (lapis_amd/loop_mapping.py decides the Kokkos level of every loop by the
 rules of the reference's loop-mapping pass and recognises that nest) is bound to the SpMV entry point, with
 its memref arguments routed by the ROLE each plays in the nest (y, positions, coordinates, values, x).
+
+Every other function made of the path's vocabulary -- `linalg.matvec` / `matmul` on CSR operands, `linalg.dot`,
+fill, copy, elementwise `linalg.generic` bodies, `tensor.*`, scalar `arith` / `math.sqrt`, `scf.while` / `for` /
+`if`, calls of private functions, and loop nests the kernel library has entry points for -- is run operation by
+operation on device-resident tensors (lapis_amd/executor.py): a CG written with other helper functions, an
+SpMV followed by an axpby, a Richardson iteration bind although no whole-function entry point exists for them.
+A function that uses anything else is refused, with the operation named.
 """
 import os
 
 import re
 
 from . import catalogue as _catalogue
+from . import executor as _executor
 from . import loop_mapping as _lm
 from . import mlir_text as _mt
 from . import module as _module
@@ -61,6 +69,85 @@ def _spmv_by_role(mod, order):
     return method
 
 
+def _run_by_operation(mod, ex, c, fname, decompose_tensors):
+    """Method for a function the executor runs operation by operation.  Arguments as the reference's wrapper
+    takes them (TranslateToKokkosCpp.cpp:2757-2977): a sparse tensor as positions, coordinates, values and the
+    specifier ((rows, columns), (len(pos), len(crd), len(val))), dense tensors and memrefs as numpy arrays,
+    scalars as Python numbers.  Tensor results come back as new numpy arrays, memref arguments are updated
+    in place; one result is returned as itself, several as a tuple."""
+    f = c.functions[fname]
+    kinds, _ = c.signature(f)
+    types = [ty for _, ty in f.args]
+
+    def method(*params, _keep=mod):
+        import numpy
+        import torch
+        params = list(params)
+        args, written = [], []
+        np_of = {"f64": numpy.float64, "f32": numpy.float32, "i32": numpy.int32, "i64": numpy.int64, "index": numpy.int64}
+
+        def up(a, elem):
+            return torch.from_numpy(numpy.ascontiguousarray(a, dtype=np_of[elem])).cuda()
+
+        def take():
+            if not params:
+                raise TypeError("@%s: too few arguments" % fname)
+            return params.pop(0)
+
+        for kind, ty in zip(kinds, types):
+            ty = ty.strip()
+            if kind.startswith("csr:"):
+                if not decompose_tensors:
+                    raise TypeError("@%s takes a sparse tensor: compile with decompose_tensors=True" % fname)
+                pos, crd, val, spec = take(), take(), take(), take()
+                args.append(_executor.Csr(up(pos, "i32"), up(crd, "i32"), up(val, kind[4:]), spec[0][0], spec[0][1]))
+            elif ty.startswith("tensor<"):
+                dims, elem = _executor._shape_spec(ty)
+                a = take()
+                args.append(up(a, elem) if dims else (numpy.float32(a) if elem == "f32" else float(a)))
+            elif ty.startswith("memref<"):
+                dims, elem = _executor._shape_spec(ty)
+                a = take()
+                if not dims:
+                    args.append(_executor.Cell(numpy.asarray(a).reshape(-1)[0]))
+                    written.append((a, args[-1]))
+                else:
+                    args.append(up(a, elem))
+                    if elem in ("f64", "f32"):
+                        written.append((a, args[-1]))
+            elif ty in ("f64", "f32"):
+                a = take()
+                args.append(numpy.float32(a) if ty == "f32" else float(a))
+            else:
+                args.append(int(take()))
+        if params:
+            raise TypeError("@%s: %d arguments too many" % (fname, len(params)))
+        try:
+            results = ex.run(fname, args)
+            out = []
+            for r in results:
+                if isinstance(r, torch.Tensor):
+                    out.append(r.cpu().numpy())
+                elif isinstance(r, _executor.Cell):
+                    out.append(r.value)
+                else:
+                    out.append(r.item() if isinstance(r, numpy.generic) and not isinstance(r, numpy.floating) else r)
+            for host, dev in written:
+                if isinstance(dev, _executor.Cell):
+                    numpy.asarray(host).reshape(-1)[0] = dev.value
+                elif isinstance(host, numpy.ndarray) and host.flags.writeable:
+                    numpy.copyto(host, dev.cpu().numpy().reshape(host.shape))
+        finally:
+            for a in args:
+                if isinstance(a, _executor.Csr):
+                    a.release()
+            ex.release()
+        if not out:
+            return None
+        return out[0] if len(out) == 1 else tuple(out)
+    return method
+
+
 class KokkosBackend:
     """Same constructor as the reference's class (python/lapis/KokkosBackend.py:13)."""
 
@@ -87,6 +174,8 @@ class KokkosBackend:
         if not public:
             raise Exception(_LOWERING_FAILED)
         bound = {}
+        self._canonicalizer = c
+        self._executor = None
         self.unbound = []
         self.loop_mapping = {}   # function name -> loop_mapping.NestMapping of a function bound at loop level
         for f in public:
@@ -101,8 +190,17 @@ class KokkosBackend:
             entry = _forms().get(form)
             if entry is None:
                 entry, why_not = self._loop_level_entry(f)
-                if entry is None and why_not:
-                    raise Exception("%s\nfunction @%s: %s" % (_LOWERING_FAILED, f.name, why_not))
+            if entry is None and (results or f.args):
+                # no whole-function entry point: operation by operation, if every operation has one
+                try:
+                    self.executor(c).check(f.name)
+                    entry = ("exec", f.name)
+                except _executor.Refused as e:
+                    if not (not results and "sparse_tensor.print" in f.body):
+                        sparse = [k for k in kinds if k.startswith("sparse(")]
+                        raise Exception("%s\nfunction @%s(%s): it uses %s%s" % (
+                            _LOWERING_FAILED, f.name, ", ".join(kinds), e,
+                            "" if not why_not else "; as one loop nest: " + why_not))
             if entry is None:
                 if not results:
                     # a helper that returns nothing (the sparse_tensor.print wrapper of examples/bspmm.py:54-58):
@@ -119,6 +217,11 @@ class KokkosBackend:
                                 "(positions, coordinates, values and the storage specifier as separate arguments)" % f.name)
             bound[method] = entry
         return bound
+
+    def executor(self, c=None):
+        if getattr(self, "_executor", None) is None:
+            self._executor = _executor.Executor(c or self._canonicalizer)
+        return self._executor
 
     def _loop_level_entry(self, f):
         """(("loops:spmv", {role: argument index}), None) when @f is one CSR SpMV loop nest over 32-bit
@@ -164,7 +267,10 @@ class KokkosBackend:
         mod = _module.LAPISModule()
         mod.bound_functions = sorted(bound)
         for method, entry in bound.items():
-            if isinstance(entry, tuple):
+            if isinstance(entry, tuple) and entry[0] == "exec":
+                setattr(mod, method, _run_by_operation(mod, self.executor(), self._canonicalizer, entry[1],
+                                                       self.decompose_tensors))
+            elif isinstance(entry, tuple):
                 setattr(mod, method, _spmv_by_role(mod, entry[1]))
             elif method != entry:
                 setattr(mod, method, getattr(mod, entry))  # the function's own name, the entry its body calls for

@@ -380,6 +380,16 @@ extern "C" int lapis_hip_fill_f32(int64_t n, float v, float *dst, lapis_hip_stre
   return launch_elementwise<float, 0>("fill_f32", n, (const float *)nullptr, (const float *)nullptr, dst,
                                       FillOp<float>{v}, as_stream(stream));
 }
+extern "C" int lapis_hip_mult_f32(int64_t n, const float *x, const float *y, float *dst, lapis_hip_stream_t stream) {
+  return launch_elementwise<float, 2>("mult_f32", n, x, y, dst, MultOp<float>{}, as_stream(stream));
+}
+extern "C" int lapis_hip_div_f32(int64_t n, const float *x, const float *y, float *dst, lapis_hip_stream_t stream) {
+  return launch_elementwise<float, 2>("div_f32", n, x, y, dst, DivOp<float>{}, as_stream(stream));
+}
+extern "C" int lapis_hip_copy_f32(int64_t n, const float *src, float *dst, lapis_hip_stream_t stream) {
+  return launch_elementwise<float, 1>("copy_f32", n, src, (const float *)nullptr, dst, CopyOp<float>{},
+                                      as_stream(stream));
+}
 extern "C" int lapis_hip_copy_f64(int64_t n, const double *src, double *dst, lapis_hip_stream_t stream) {
   return launch_elementwise<double, 1>("copy_f64", n, src, (const double *)nullptr, dst, CopyOp<double>{},
                                        as_stream(stream));

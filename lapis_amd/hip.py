@@ -88,10 +88,13 @@ _SIGNATURES = {
     "lapis_hip_axpby_f64": [_i64, _dbl, _vp, _dbl, _vp, _vp, _vp],
     "lapis_hip_axpby_f32": [_i64, _flt, _vp, _flt, _vp, _vp, _vp],
     "lapis_hip_mult_f64": [_i64, _vp, _vp, _vp, _vp],
+    "lapis_hip_mult_f32": [_i64, _vp, _vp, _vp, _vp],
     "lapis_hip_div_f64": [_i64, _vp, _vp, _vp, _vp],
+    "lapis_hip_div_f32": [_i64, _vp, _vp, _vp, _vp],
     "lapis_hip_fill_f64": [_i64, _dbl, _vp, _vp],
     "lapis_hip_fill_f32": [_i64, _flt, _vp, _vp],
     "lapis_hip_copy_f64": [_i64, _vp, _vp, _vp],
+    "lapis_hip_copy_f32": [_i64, _vp, _vp, _vp],
     "lapis_hip_scale_f64": [_i64, _dbl, _vp, _vp],
     "lapis_hip_pcg_masked_f64_i32": [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _dbl, _u64, _vp,
                                      ctypes.POINTER(_u64), ctypes.POINTER(_dbl), _vp, _vp],
@@ -370,12 +373,12 @@ def axpby(a, x, b, y, dst, stream=None):
 
 
 def mult(x, y, dst, stream=None):
-    check(init().lapis_hip_mult_f64(int(x.shape[0]), _ptr(x), _ptr(y), _ptr(dst), _stream(stream)))
+    check(getattr(init(), "lapis_hip_mult_%s" % _suffix(x))(int(x.shape[0]), _ptr(x), _ptr(y), _ptr(dst), _stream(stream)))
     return dst
 
 
 def div(x, y, dst, stream=None):
-    check(init().lapis_hip_div_f64(int(x.shape[0]), _ptr(x), _ptr(y), _ptr(dst), _stream(stream)))
+    check(getattr(init(), "lapis_hip_div_%s" % _suffix(x))(int(x.shape[0]), _ptr(x), _ptr(y), _ptr(dst), _stream(stream)))
     return dst
 
 
@@ -387,7 +390,7 @@ def fill(dst, value, stream=None):
 
 
 def copy(src, dst, stream=None):
-    check(init().lapis_hip_copy_f64(int(src.shape[0]), _ptr(src), _ptr(dst), _stream(stream)))
+    check(getattr(init(), "lapis_hip_copy_%s" % _suffix(src))(int(src.shape[0]), _ptr(src), _ptr(dst), _stream(stream)))
     return dst
 
 

@@ -164,3 +164,108 @@ module {
 """
 
 SHAPES = {"loop_mapping_0": HOST_2D, "loop_mapping_1": COUNT, "loop_mapping_2": SPMV_INDEX, "loop_mapping_3": DEEP4}
+
+
+# ---- depth-1 loops and the SpMM nest the kernel library has entry points for ------------------------------
+
+# a dot product as DenseLinalgToParallelLoops leaves it (the shape of linalg_to_loops_0's gold): the reduction
+# starts from the value of a zero-dimensional buffer, which gets the result
+DOT = """
+module {
+  func.func @inner(%u: memref<?xf64>, %v: memref<?xf64>, %start: f64) -> f64 {
+    %zero = arith.constant 0 : index
+    %one = arith.constant 1 : index
+    %cell = memref.alloc() {alignment = 64 : i64} : memref<f64>
+    memref.store %start, %cell[] : memref<f64>
+    %count = memref.dim %u, %zero : memref<?xf64>
+    %from = memref.load %cell[] : memref<f64>
+    %total = scf.parallel (%k) = (%zero) to (%count) step (%one) init (%from) -> f64 {
+      %a = memref.load %u[%k] : memref<?xf64>
+      %b = memref.load %v[%k] : memref<?xf64>
+      %prod = arith.mulf %a, %b : f64
+      scf.reduce(%prod : f64) {
+      ^bb0(%lhs: f64, %rhs: f64):
+        %s = arith.addf %lhs, %rhs : f64
+        scf.reduce.return %s : f64
+      }
+    }
+    memref.store %total, %cell[] : memref<f64>
+    %got = memref.load %cell[] : memref<f64>
+    return %got : f64
+  }
+}
+"""
+
+# the same loop with a product reduction: no entry point
+DOT_PRODUCT_REDUCTION = DOT.replace("%s = arith.addf %lhs, %rhs", "%s = arith.mulf %lhs, %rhs")
+
+
+def elementwise(body, elem="f64", name="update"):
+    """A depth-1 loop `w[k] = <body>(u[k], v[k], p, q)`; `body` defines %r from %a, %b, %p, %q."""
+    return """
+module {
+  func.func @%(name)s(%%p: %(t)s, %%u: memref<?x%(t)s>, %%q: %(t)s, %%v: memref<?x%(t)s>, %%w: memref<?x%(t)s>) {
+    %%zero = arith.constant 0 : index
+    %%one = arith.constant 1 : index
+    %%count = memref.dim %%w, %%zero : memref<?x%(t)s>
+    scf.parallel (%%k) = (%%zero) to (%%count) step (%%one) {
+      %%a = memref.load %%u[%%k] : memref<?x%(t)s>
+      %%b = memref.load %%v[%%k] : memref<?x%(t)s>
+%(body)s
+      memref.store %%r, %%w[%%k] : memref<?x%(t)s>
+      scf.reduce
+    }
+    return
+  }
+}
+""" % {"t": elem, "name": name, "body": body.replace("%", "%%").replace("%%", "%") % {"t": elem} if "%(t)s" in body else body}
+
+
+AXPBY_BODY = """      %l = arith.mulf %a, %p : f64
+      %m = arith.mulf %b, %q : f64
+      %r = arith.addf %l, %m : f64"""
+MULT_BODY = "      %r = arith.mulf %a, %b : f64"
+SCALE_BODY = "      %r = arith.mulf %p, %a : f64"
+FILL_BODY = "      %r = arith.addf %p, %q : f64"
+CUBE_BODY = """      %l = arith.mulf %a, %a : f64
+      %r = arith.mulf %l, %b : f64"""
+
+
+def spmm_i32(elem="f32", inner="scf.parallel", name="rows_times_dense"):
+    """C[i, j] += sum_kk val[kk] * B[crd[kk], j]: rows parallel, the compressed loop sequential, the dense column
+    loop parallel (`inner="scf.parallel"`) or sequential (`inner="scf.for"`)."""
+    if inner == "scf.parallel":
+        open_j, close_j = "scf.parallel (%j) = (%zero) to (%cols) step (%one) {", "          scf.reduce\n        }"
+    else:
+        open_j, close_j = "scf.for %j = %zero to %cols step %one {", "        }"
+    return """
+module {
+  func.func @%(name)s(%%B: memref<?x?x%(t)s>, %%ptr: memref<?xi32>, %%idx: memref<?xi32>, %%C: memref<?x?x%(t)s>, %%nz: memref<?x%(t)s>) {
+    %%zero = arith.constant 0 : index
+    %%one = arith.constant 1 : index
+    %%rows = memref.dim %%C, %%zero : memref<?x?x%(t)s>
+    %%cols = memref.dim %%C, %%one : memref<?x?x%(t)s>
+    scf.parallel (%%i) = (%%zero) to (%%rows) step (%%one) {
+      %%lo32 = memref.load %%ptr[%%i] : memref<?xi32>
+      %%lo = arith.index_cast %%lo32 : i32 to index
+      %%inext = arith.addi %%i, %%one : index
+      %%hi32 = memref.load %%ptr[%%inext] : memref<?xi32>
+      %%hi = arith.index_cast %%hi32 : i32 to index
+      scf.for %%kk = %%lo to %%hi step %%one {
+        %%c32 = memref.load %%idx[%%kk] : memref<?xi32>
+        %%c = arith.index_cast %%c32 : i32 to index
+        %%a = memref.load %%nz[%%kk] : memref<?x%(t)s>
+        %(open_j)s
+          %%old = memref.load %%C[%%i, %%j] : memref<?x?x%(t)s>
+          %%b = memref.load %%B[%%c, %%j] : memref<?x?x%(t)s>
+          %%prod = arith.mulf %%a, %%b : %(t)s
+          %%new = arith.addf %%old, %%prod : %(t)s
+          memref.store %%new, %%C[%%i, %%j] : memref<?x?x%(t)s>
+%(close_j)s
+      }
+      scf.reduce
+    }
+    return
+  }
+}
+""" % {"t": elem, "name": name, "open_j": open_j.replace("%", "%%").replace("%%", "%"), "close_j": close_j}

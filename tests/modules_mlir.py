@@ -164,3 +164,172 @@ module {
     return
   }
 }"""
+
+# ---- functions no whole-function entry point exists for: bound operation by operation ----------------------
+
+# an SpMV followed by an axpby: alpha * (A x) + beta * z
+SPMV_THEN_AXPBY = """
+#CSR = #sparse_tensor.encoding<{ map = (d0, d1) -> (d0 : dense, d1 : compressed), posWidth = 32, crdWidth = 32 }>
+#id = affine_map<(d0) -> (d0)>
+module {
+  func.func @residual(%A: tensor<?x?xf64, #CSR>, %x: tensor<?xf64>, %z: tensor<?xf64>, %alpha: f64, %beta: f64) -> tensor<?xf64> {
+    %c0 = arith.constant 0 : index
+    %rows = tensor.dim %A, %c0 : tensor<?x?xf64, #CSR>
+    %f0 = arith.constant 0.0 : f64
+    %e = tensor.empty(%rows) : tensor<?xf64>
+    %clean = linalg.fill ins(%f0 : f64) outs(%e : tensor<?xf64>) -> tensor<?xf64>
+    %Ax = linalg.matvec ins(%A, %x : tensor<?x?xf64, #CSR>, tensor<?xf64>) outs(%clean : tensor<?xf64>) -> tensor<?xf64>
+    %e2 = tensor.empty(%rows) : tensor<?xf64>
+    %out = linalg.generic {indexing_maps = [#id, #id, #id], iterator_types = ["parallel"]}
+        ins(%Ax, %z : tensor<?xf64>, tensor<?xf64>) outs(%e2 : tensor<?xf64>) {
+      ^bb0(%a: f64, %b: f64, %o: f64):
+        %l = arith.mulf %alpha, %a : f64
+        %m = arith.mulf %beta, %b : f64
+        %s = arith.addf %l, %m : f64
+        linalg.yield %s : f64
+    } -> tensor<?xf64>
+    return %out : tensor<?xf64>
+  }
+}"""
+
+# unpreconditioned CG from x = 0 whose residual update r - alpha*Ap is ONE generic with a subtraction, and whose
+# direction update reads its own output operand
+CG_FUSED_UPDATE = """
+#CSR = #sparse_tensor.encoding<{ map = (d0, d1) -> (d0 : dense, d1 : compressed), posWidth = 32, crdWidth = 32 }>
+#id = affine_map<(d0) -> (d0)>
+module {
+  func.func private @inner(%a: tensor<?xf64>, %b: tensor<?xf64>) -> f64 {
+    %c = arith.constant 0.0 : f64
+    %acc = tensor.splat %c[] : tensor<f64>
+    %d = linalg.dot ins(%a, %b : tensor<?xf64>, tensor<?xf64>) outs(%acc : tensor<f64>) -> tensor<f64>
+    %s = tensor.extract %d[] : tensor<f64>
+    return %s : f64
+  }
+  func.func @cg(%A: tensor<?x?xf64, #CSR>, %b: tensor<?xf64>, %tol: f64, %maxiter: index) -> (tensor<?xf64>, index, f64) {
+    %c0 = arith.constant 0 : index
+    %c1 = arith.constant 1 : index
+    %f0 = arith.constant 0.0 : f64
+    %n = tensor.dim %b, %c0 : tensor<?xf64>
+    %x0 = tensor.splat %f0[%n] : tensor<?xf64>
+    %e0 = tensor.empty(%n) : tensor<?xf64>
+    %p0 = linalg.copy ins(%b : tensor<?xf64>) outs(%e0 : tensor<?xf64>) -> tensor<?xf64>
+    %bb = func.call @inner(%b, %b) : (tensor<?xf64>, tensor<?xf64>) -> f64
+    %bnorm = math.sqrt %bb : f64
+    %x, %r, %p, %rr, %its = scf.while (%xi = %x0, %ri = %b, %pi = %p0, %rri = %bb, %i = %c0)
+        : (tensor<?xf64>, tensor<?xf64>, tensor<?xf64>, f64, index) -> (tensor<?xf64>, tensor<?xf64>, tensor<?xf64>, f64, index) {
+      %nrm = math.sqrt %rri : f64
+      %rel = arith.divf %nrm, %bnorm : f64
+      %open = arith.cmpf ogt, %rel, %tol : f64
+      %more = arith.cmpi slt, %i, %maxiter : index
+      %go = arith.andi %open, %more : i1
+      scf.condition(%go) %xi, %ri, %pi, %rri, %i : tensor<?xf64>, tensor<?xf64>, tensor<?xf64>, f64, index
+    } do {
+    ^bb0(%xi: tensor<?xf64>, %ri: tensor<?xf64>, %pi: tensor<?xf64>, %rri: f64, %i: index):
+      %e1 = tensor.empty(%n) : tensor<?xf64>
+      %z = linalg.fill ins(%f0 : f64) outs(%e1 : tensor<?xf64>) -> tensor<?xf64>
+      %Ap = linalg.matvec ins(%A, %pi : tensor<?x?xf64, #CSR>, tensor<?xf64>) outs(%z : tensor<?xf64>) -> tensor<?xf64>
+      %pAp = func.call @inner(%pi, %Ap) : (tensor<?xf64>, tensor<?xf64>) -> f64
+      %alpha = arith.divf %rri, %pAp : f64
+      %xn = linalg.generic {indexing_maps = [#id, #id], iterator_types = ["parallel"]}
+          ins(%pi : tensor<?xf64>) outs(%xi : tensor<?xf64>) {
+        ^bb0(%pe: f64, %xe: f64):
+          %t = arith.mulf %alpha, %pe : f64
+          %u = arith.addf %xe, %t : f64
+          linalg.yield %u : f64
+      } -> tensor<?xf64>
+      %rn = linalg.generic {indexing_maps = [#id, #id, #id], iterator_types = ["parallel"]}
+          ins(%ri, %Ap : tensor<?xf64>, tensor<?xf64>) outs(%e1 : tensor<?xf64>) {
+        ^bb0(%re: f64, %ae: f64, %oe: f64):
+          %t = arith.mulf %alpha, %ae : f64
+          %u = arith.subf %re, %t : f64
+          linalg.yield %u : f64
+      } -> tensor<?xf64>
+      %rrn = func.call @inner(%rn, %rn) : (tensor<?xf64>, tensor<?xf64>) -> f64
+      %beta = arith.divf %rrn, %rri : f64
+      %pn = linalg.generic {indexing_maps = [#id, #id], iterator_types = ["parallel"]}
+          ins(%rn : tensor<?xf64>) outs(%pi : tensor<?xf64>) {
+        ^bb0(%re: f64, %pe: f64):
+          %t = arith.mulf %beta, %pe : f64
+          %u = arith.addf %re, %t : f64
+          linalg.yield %u : f64
+      } -> tensor<?xf64>
+      %in = arith.addi %i, %c1 : index
+      scf.yield %xn, %rn, %pn, %rrn, %in : tensor<?xf64>, tensor<?xf64>, tensor<?xf64>, f64, index
+    }
+    %nrm = math.sqrt %rr : f64
+    %relres = arith.divf %nrm, %bnorm : f64
+    return %x, %its, %relres : tensor<?xf64>, index, f64
+  }
+}"""
+
+# Richardson iteration x <- x + omega (b - A x), a fixed number of sweeps, with named elementwise operations
+RICHARDSON = """
+#CSR = #sparse_tensor.encoding<{ map = (d0, d1) -> (d0 : dense, d1 : compressed), posWidth = 32, crdWidth = 32 }>
+#id = affine_map<(d0) -> (d0)>
+module {
+  func.func @richardson(%A: tensor<?x?xf64, #CSR>, %b: tensor<?xf64>, %x0: tensor<?xf64>, %omega: f64, %sweeps: index) -> tensor<?xf64> {
+    %c0 = arith.constant 0 : index
+    %c1 = arith.constant 1 : index
+    %f0 = arith.constant 0.0 : f64
+    %n = tensor.dim %b, %c0 : tensor<?xf64>
+    %x = scf.for %k = %c0 to %sweeps step %c1 iter_args(%xk = %x0) -> (tensor<?xf64>) {
+      %e = tensor.empty(%n) : tensor<?xf64>
+      %z = linalg.fill ins(%f0 : f64) outs(%e : tensor<?xf64>) -> tensor<?xf64>
+      %Ax = linalg.matvec ins(%A, %xk : tensor<?x?xf64, #CSR>, tensor<?xf64>) outs(%z : tensor<?xf64>) -> tensor<?xf64>
+      %e2 = tensor.empty(%n) : tensor<?xf64>
+      %res = linalg.sub ins(%b, %Ax : tensor<?xf64>, tensor<?xf64>) outs(%e2 : tensor<?xf64>) -> tensor<?xf64>
+      %e3 = tensor.empty(%n) : tensor<?xf64>
+      %xn = linalg.generic {indexing_maps = [#id, #id, #id], iterator_types = ["parallel"]}
+          ins(%xk, %res : tensor<?xf64>, tensor<?xf64>) outs(%e3 : tensor<?xf64>) {
+        ^bb0(%xe: f64, %re: f64, %oe: f64):
+          %t = arith.mulf %omega, %re : f64
+          %u = arith.addf %xe, %t : f64
+          linalg.yield %u : f64
+      } -> tensor<?xf64>
+      scf.yield %xn : tensor<?xf64>
+    }
+    return %x : tensor<?xf64>
+  }
+}"""
+
+# two products in a row, y = A (A x), and a function whose operand it must not overwrite: %x is used again
+TWO_PRODUCTS = """
+#CSR = #sparse_tensor.encoding<{ map = (d0, d1) -> (d0 : dense, d1 : compressed), posWidth = 32, crdWidth = 32 }>
+module {
+  func.func @twice_plus(%A: tensor<?x?xf64, #CSR>, %x: tensor<?xf64>) -> (tensor<?xf64>, tensor<?xf64>) {
+    %Ax = linalg.matvec ins(%A, %x : tensor<?x?xf64, #CSR>, tensor<?xf64>) outs(%x : tensor<?xf64>) -> tensor<?xf64>
+    %AAx = linalg.matvec ins(%A, %Ax : tensor<?x?xf64, #CSR>, tensor<?xf64>) outs(%x : tensor<?xf64>) -> tensor<?xf64>
+    return %Ax, %AAx : tensor<?xf64>, tensor<?xf64>
+  }
+}"""
+
+# the CSR x dense product written as a generic (the form of examples/spmm_dcsr_opdsl.py), scaled afterwards
+SPMM_GENERIC_SCALED = """
+#CSR = #sparse_tensor.encoding<{ map = (d0, d1) -> (d0 : dense, d1 : compressed), posWidth = 32, crdWidth = 32 }>
+#id2 = affine_map<(d0, d1) -> (d0, d1)>
+module {
+  func.func @scaled_product(%A: tensor<?x?xf32, #CSR>, %B: tensor<?x?xf32>, %C: tensor<?x?xf32>, %s: f32) -> tensor<?x?xf32> {
+    %AB = linalg.generic {
+        indexing_maps = [affine_map<(i, j, k) -> (i, k)>, affine_map<(i, j, k) -> (k, j)>, affine_map<(i, j, k) -> (i, j)>],
+        iterator_types = ["parallel", "parallel", "reduction"]}
+        ins(%A, %B : tensor<?x?xf32, #CSR>, tensor<?x?xf32>) outs(%C : tensor<?x?xf32>) {
+      ^bb0(%a: f32, %b: f32, %c: f32):
+        %p = arith.mulf %a, %b : f32
+        %q = arith.addf %c, %p : f32
+        linalg.yield %q : f32
+    } -> tensor<?x?xf32>
+    %out = linalg.generic {indexing_maps = [#id2, #id2], iterator_types = ["parallel", "parallel"]}
+        ins(%AB : tensor<?x?xf32>) outs(%AB : tensor<?x?xf32>) {
+      ^bb0(%e: f32, %o: f32):
+        %t = arith.mulf %e, %s : f32
+        linalg.yield %t : f32
+    } -> tensor<?x?xf32>
+    return %out : tensor<?x?xf32>
+  }
+}"""
+
+# the same conjugate gradients in single precision
+PCG_F32 = PCG.replace("f64", "f32")
+
+# an operation outside the vocabulary between two that are inside it
+SPMV_THEN_EXP = SPMV_THEN_AXPBY.replace("%s = arith.addf %l, %m : f64", "%s0 = arith.addf %l, %m : f64\n        %s = math.exp %s0 : f64")
