@@ -1,10 +1,11 @@
-// RUN: %lapis-translate --hip-kernels %s | grep -E -c "KOKKOS_LAMBDA|lapis_hip_spmv_csr_f64_i32\(lapis_hip_plan_|lapis_hip_csr_plan_create\(&lapis_hip_plan_|lapis_hip_csr_plan_destroy\(lapis_hip_plan_|lapis_hip_init\(\)|lapis_hip_finalize\(\)" | diff %s.gold -
+// RUN: %lapis-translate --hip-kernels %s | grep -E -c "KOKKOS_LAMBDA|lapis_hip_spmv_csr_f64_i32\(lapis_hip_plan_|lapis_hip_csr_plan_create\(&lapis_hip_plan_|lapis_hip_csr_plan_matches\(lapis_hip_plan_|lapis_hip_csr_plan_analyze\(lapis_hip_plan_|lapis_hip_csr_plan_destroy\(lapis_hip_plan_|lapis_hip_init\(\)|lapis_hip_finalize\(\)" | diff %s.gold -
 
-// The mapped CSR SpMV nest (hip_spmv_0.mlir.gold) translated with --hip-kernels: one call of
-// lapis_hip_spmv_csr_f64_i32 (tried with the kept plan, repeated after the plan is (re)built: 2 lines),
-// one lapis_hip_csr_plan_create, lapis_hip_csr_plan_destroy before the rebuild and in lapis_finalize
-// (2 lines), lapis_hip_init in lapis_initialize, lapis_hip_finalize in lapis_finalize -- and no
-// KOKKOS_LAMBDA: 7 matching lines.
+// The mapped CSR SpMV nest (hip_spmv_0.mlir.gold) translated with --hip-kernels: the kept plan is checked
+// against the operands (lapis_hip_csr_plan_matches and the generation of the operands, 1 line) and
+// destroyed if it was made for others, created if there is none (lapis_hip_csr_plan_create), then ONE call
+// of lapis_hip_spmv_csr_f64_i32; lapis_hip_csr_plan_destroy before the rebuild and in lapis_finalize
+// (2 lines), lapis_hip_init in lapis_initialize, lapis_hip_finalize in lapis_finalize -- no
+// lapis_hip_csr_plan_analyze (the nest is not inside a loop) and no KOKKOS_LAMBDA: 7 matching lines.
 module {
   func.func @spmv(%arg0: memref<?xf64>, %arg1: memref<?xi32>, %arg2: memref<?xi32>, %arg3: memref<?xf64>, %arg4: memref<?xf64>) {
     %c0 = arith.constant 0 : index
