@@ -404,6 +404,17 @@ def run_spmm(args):
         if k != B.shape[1]:
             B = gen.uniform_matrix(A.ncols, k, 4005).astype(np.float32)
         name = "config4: SpMM fp32, A 1048576^2 with 32 nnz/row, B 1048576x%d row-major" % k
+        if args.spmm_fold_b:
+            # the same matrix with its columns folded onto the first R rows of B: what the kernel would cost if B
+            # were that much smaller (the most that blocking B could buy)
+            R = args.spmm_fold_b
+            crd = (A.crd % R).astype(np.int32)
+            rows = np.repeat(np.arange(A.nrows, dtype=np.int64), np.diff(A.pos))
+            order = np.lexsort((crd, rows))
+            A = gen.CSR(A.nrows, R, A.pos, crd[order], A.val[order])
+            B = np.ascontiguousarray(B[:R])
+            name = "config4 with the columns of A folded onto %d rows of B (%d x %d fp32, %.1f MB)" % (
+                R, R, k, R * k * 4 / 1e6)
     dev = lambda a: torch.from_numpy(a).cuda()
     pos, crd, val, dB = dev(A.pos), dev(A.crd), dev(A.val), dev(B)
     C = torch.zeros(A.nrows, k, dtype=torch.float32, device="cuda")
@@ -437,7 +448,7 @@ def run_spmm(args):
         "roofline": {"bound": "hbm", "kernel": "%s<float>" % hip.spmm_last_kernel(), "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": traffic_from_profiles("spmm_config4", kt["mean_ms"])
-                     if not args.workload and k == 64 else None,
+                     if not args.workload and k == 64 and not args.spmm_fold_b else None,
                      "traffic_source": TRAFFIC_SOURCE,
                      "kernel_ms_mean": kt["mean_ms"], "kernel_ms_median": kt["median_ms"],
                      "kernel_ms_min": kt["min_ms"], "launches_timed": kt["count"]},
@@ -531,6 +542,9 @@ def main():
                     help="layout of the column-blocked copy (auto = group)")
     ap.add_argument("--width", type=int, default=0, help="lanes per row with --kernel subwarp (0 = the reference's rule)")
     ap.add_argument("--k", type=int, default=64, help="columns of B for the SpMM workloads (config 4)")
+    ap.add_argument("--spmm-fold-b", type=int, default=0,
+                    help="config 4 with the column indices of A taken modulo this many rows of B (an experiment: "
+                         "what a smaller B would cost)")
     ap.add_argument("--spmm-kernel", choices=["auto", "wave", "group", "lds"], default="auto",
                     help="SpMM kernel: the plan's choice, the wavefront-per-row kernel, or the LDS-staged row-block kernel")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -591,6 +605,7 @@ def run_others(args):
         a = copy.copy(args)
         a.config, a.no_cpu, a.no_calibration, a.graph, a.host_buffers = cfg, True, True, False, False
         a.kernel, a.workload, a.k, a.spmm_kernel = None, None, 64, "auto"
+        a.spmm_fold_b = 0
         a.steps, a.warmup = min(20, {3: 20, 4: 20, 5: 20}[cfg]), 2
         gc.collect()
         torch.cuda.empty_cache()
