@@ -266,6 +266,13 @@ class KokkosBackend:
         bound = self.bind(moduleText)
         mod = _module.LAPISModule()
         mod.bound_functions = sorted(bound)
+        # python/lapis/KokkosBackend.py:21-24,113-114: the package of instance k is lapis_package_k, and only the
+        # last of `num_instances` modules is emitted with --finalize (it shuts Kokkos down).  Here every module
+        # shares one prebuilt library whose lapis_initialize / lapis_finalize count the live modules, so the
+        # runtime goes down with the last module whichever index it has; the two attributes record what the
+        # reference would have generated.
+        mod.package_name = self.package_name
+        mod.finalizes_runtime = self.num_instances == 0 or self.index_instance == self.num_instances - 1
         for method, entry in bound.items():
             if isinstance(entry, tuple) and entry[0] == "exec":
                 setattr(mod, method, _run_by_operation(mod, self.executor(), self._canonicalizer, entry[1],

@@ -357,8 +357,10 @@ __global__ __launch_bounds__(256) void band_stats_kernel(int nrows, long long nn
   const long long r = (long long)blockIdx.x * 256 + threadIdx.x;
   unsigned cnt[4] = {0u, 0u, 0u, 0u};
   if (r < nrows) {
-    // the structure has not been validated yet: stay inside crd whatever pos holds
-    const long long first = std::max<long long>(0, pos[r]), last = std::min<long long>(nnz, pos[r + 1]);
+    // the structure has not been validated yet: stay inside crd whatever pos holds, and spend nothing on a
+    // row whose positions decrease (the plan is refused for it anyway)
+    const long long first = std::max<long long>(0, pos[r]);
+    const long long last = pos[r + 1] < pos[r] ? first : std::min<long long>(nnz, pos[r + 1]);
     for (long long j = first; j < last; ++j) {
       const long long d = (long long)crd[j] - r;
       const long long a = d < 0 ? -d : d;

@@ -249,6 +249,17 @@ def test_two_modules_share_the_library_and_outlive_each_other(gpu, golden):
     second.spmv(rowptrs, colinds, values, ((5, 5), (6, 8, 8)), np.ones(5), y)  # the library is still initialised
     assert np.allclose(y, g["y_expected"])
     del junk
+    # the packaging arguments of examples/twomodules.py:36-39: instance k is package lapis_package_k and only the
+    # last instance would have been emitted with --finalize; both run whichever goes first
+    k1 = KokkosBackend.KokkosBackend(decompose_tensors=True, index_instance=0, num_instances=2).compile(M.SPMV)
+    k2 = KokkosBackend.KokkosBackend(decompose_tensors=True, index_instance=1, num_instances=2).compile(M.MATVEC_OTHER_NAME)
+    assert (k1.package_name, k1.finalizes_runtime) == ("lapis_package", False)
+    assert (k2.package_name, k2.finalizes_runtime) == ("lapis_package_1", True)
+    del k2  # the "finalizing" module goes first: the other one still runs
+    gc.collect()
+    y = np.zeros(5)
+    k1.spmv(rowptrs, colinds, values, ((5, 5), (6, 8, 8)), np.ones(5), y)
+    assert np.allclose(y, g["y_expected"])
 
 
 # ---- operands that stay on the device -----------------------------------------------------------------
