@@ -525,6 +525,28 @@ def run_cg(args):
         dt = (time.perf_counter() - t0) / reps
         out["cpu_baseline"] = {"value": bytes_step / dt / 1e9, "unit": "GB/s", "cores": omp.max_threads(), "kind": "port",
                                "sample": "%d iterations' worth of SpMV + 2 dots + 3 axpy on the full workload" % reps}
+    if args.module:
+        # the same solve through the generated-module boundary: py_pcg copies every operand per call, the
+        # resident handles keep the matrix and the vectors on the device
+        from lapis_amd.module import LAPISModule
+        del pos, crd, val, db, x, work
+        torch.cuda.empty_cache()
+        mod = LAPISModule()
+        spec = ((n, n), (n + 1, A.nnz, A.nnz))
+        t0 = time.perf_counter()
+        _, it, _ = mod.pcg(A.pos, A.crd, A.val, spec, b, np.ones(n), 0.0, args.steps)
+        per_call = time.perf_counter() - t0
+        Ad = mod.bind_csr(A.pos, A.crd, A.val, spec)
+        bv, xv = mod.dual_view(b), mod.dual_view(np.zeros(n))
+        Ad.pcg(bv, None, 0.0, 2, xv)
+        t0 = time.perf_counter()
+        _, it2, _ = Ad.pcg(bv, None, 0.0, args.steps, xv)
+        resident = time.perf_counter() - t0
+        out["through_module"] = {
+            "py_pcg_ms_per_call": per_call * 1e3, "py_pcg_iterations": int(it),
+            "py_pcg_note": "host operands copied in and out by the call, Jacobi preconditioner of ones",
+            "resident_ms_per_iteration": resident / args.steps * 1e3, "resident_iterations": int(it2),
+            "resident_GB_per_s": bytes_step / (resident / args.steps) / 1e9}
     return out
 
 
@@ -556,6 +578,9 @@ def main():
                     help="print the whole gather/stream calibration table (merge factors, cache levels) instead of "
                          "the three rows the secondary roofline needs")
     ap.add_argument("--no-calibration", action="store_true", help="skip the gather/stream calibration launches")
+    ap.add_argument("--module", action="store_true",
+                    help="config 5: also run the solve through the generated-module boundary (py_pcg with host "
+                         "operands, and the device-resident handles)")
     ap.add_argument("--no-others", action="store_true",
                     help="with the default configuration: do not also run configurations 3, 4 and 5 (the 'others' block)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -605,7 +630,7 @@ def run_others(args):
         a = copy.copy(args)
         a.config, a.no_cpu, a.no_calibration, a.graph, a.host_buffers = cfg, True, True, False, False
         a.kernel, a.workload, a.k, a.spmm_kernel = None, None, 64, "auto"
-        a.spmm_fold_b = 0
+        a.spmm_fold_b, a.module = 0, False
         a.steps, a.warmup = min(20, {3: 20, 4: 20, 5: 20}[cfg]), 2
         gc.collect()
         torch.cuda.empty_cache()
