@@ -87,7 +87,7 @@ def _run_by_operation(mod, ex, c, fname, decompose_tensors):
         np_of = {"f64": numpy.float64, "f32": numpy.float32, "i32": numpy.int32, "i64": numpy.int64, "index": numpy.int64}
 
         def up(a, elem):
-            return torch.from_numpy(numpy.ascontiguousarray(a, dtype=np_of[elem])).cuda()
+            return torch.from_numpy(numpy.array(a, dtype=np_of[elem], order="C")).to(ex.device)
 
         def take():
             if not params:

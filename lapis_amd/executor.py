@@ -152,7 +152,10 @@ def _mentions(stmt, out):
 
 
 class Executor:
-    def __init__(self, canonicalizer, torch_module=None, hip_module=None):
+    def __init__(self, canonicalizer, torch_module=None, hip_module=None, device="cuda"):
+        # `hip_module` / `device`: the tests of the host logic pass a stand-in for lapis_amd.hip that works on
+        # CPU tensors; the product never does (KokkosBackend constructs Executor(canonicalizer))
+        self.device = device
         self.c = canonicalizer
         self.aliases = canonicalizer.aliases
         self._parsed = {}
@@ -473,7 +476,7 @@ class Executor:
     def _new(self, shape, elem):
         torch = self.torch
         return torch.empty(tuple(int(d) for d in shape), dtype=torch.float64 if elem == "f64" else
-                           torch.float32 if elem == "f32" else torch.int32, device="cuda")
+                           torch.float32 if elem == "f32" else torch.int32, device=self.device)
 
     def _sizes(self, ty, dynamic):
         dims, elem = _shape_spec(ty)
@@ -563,7 +566,7 @@ class Executor:
             idx = [self._val(env, n) for n in names[1:]]
             if isinstance(t, Cell):
                 return [t.value]
-            if not hasattr(t, "shape"):
+            if not isinstance(t, torch.Tensor):  # a zero-dimensional tensor is kept as a host scalar
                 return [t]
             v = t[tuple(idx)].item()  # waits for the kernels that produce it
             return [numpy.float32(v) if t.dtype == torch.float32 else v]
@@ -590,7 +593,7 @@ class Executor:
             raise Refused("%s with %d outputs" % (op, len(outs)))
         out_nm = outs[0]
         out_v = self._val(env, out_nm)
-        scalar_out = not hasattr(out_v, "shape")  # a zero-dimensional tensor (host scalar) or a Cell
+        scalar_out = not isinstance(out_v, torch.Tensor)  # a zero-dimensional tensor (host scalar) or a Cell
         in_vals = [self._val(env, n) for n in ins]
         in_place = not result_is_tensor  # memref semantics
         flat = lambda t: t.reshape(-1)
