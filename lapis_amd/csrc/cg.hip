@@ -18,6 +18,11 @@
 // kernel cost more than the vector pass itself).  The iteration number is a kernel
 // argument (the host knows which iteration it is queueing); scalars that one kernel
 // both reads and replaces (r.z) are kept twice, indexed by iteration parity.
+//
+// x is needed by nobody until the solve ends, so x += alpha p is made by the kernel
+// that reads p anyway to replace it (p = z + beta p), not by the one that updates r:
+// p is then read twice per iteration (by the SpMV's gathers and by that kernel), not
+// three times.  The pass that decides to leave still adds its alpha p and leaves p alone.
 #include <algorithm>
 #include <cmath>
 
@@ -34,10 +39,10 @@ struct CgState {
   double rr;       // r . r after the update
   double initres;  // sqrt(r0 . r0)
   double relres;
-  unsigned long long iter;  // the reference's counter i at exit (it starts at 1)
+  double alpha;    // r.z / p.Ap of the iteration under way
+  unsigned long long done_iter;  // 0 while iterating, then the reference's counter i at exit (it starts at 1)
   unsigned long long maxiter;
   double tol;
-  int done;
 };
 
 __device__ __forceinline__ double block_sum_256d(double v, double *lds4) {
@@ -49,14 +54,14 @@ __device__ __forceinline__ double block_sum_256d(double v, double *lds4) {
   return total;
 }
 
-// The exit flag, read once per block: block 0 of the kernel that makes the convergence
-// test raises it while other blocks of the same kernel may still be starting, and
+// The exit mark, read once per block: block 0 of the kernel that makes the convergence
+// test sets it while other blocks of the same kernel may still be starting, and
 // every thread of a block has to take the same way past the barriers below.
-__device__ __forceinline__ bool block_sees_done(const CgState *st) {
-  __shared__ int seen;
-  if (threadIdx.x == 0) seen = st->done;
+__device__ __forceinline__ unsigned long long block_done_iter(const CgState *st) {
+  __shared__ unsigned long long seen;
+  if (threadIdx.x == 0) seen = st->done_iter;
   __syncthreads();
-  const bool d = seen != 0;
+  const unsigned long long d = seen;
   __syncthreads();
   return d;
 }
@@ -120,97 +125,73 @@ __global__ __launch_bounds__(256) void cg_pap_kernel(long long n, const double *
   if (threadIdx.x == 0) partials[blockIdx.x] = bsum;
 }
 
-// The same partials when Ap came from the row-split SpMV kernel with its fix-up left out:
-// a block takes `rows_per_block` consecutive rows (an even number, so the 128-bit accesses
-// stay aligned), first completes the rows of its range that are cut at chunk boundaries
-// (boundaries block_c[b] .. block_c[b+1]-1), then sums.  Only this block reads those rows
-// in this kernel, so a workgroup barrier orders the completion before the sum.
+// The same partials when Ap came from the row-split SpMV kernel with its fix-up left out
+// and the chunk sums of p[r]*Ap[r] over uncut rows taken (`chunk_pap`): thread t of a
+// block completes the row cut at chunk boundary c (if that boundary is the first to cut
+// it), adds that row's p[r]*Ap[r], and adds chunk c's sum.  Neither vector is read in
+// full again.  Chunks and boundaries are dealt to blocks and lanes in a fixed order.
 template <int CH>
-__global__ __launch_bounds__(256) void cg_pap_fix_kernel(long long n, long long rows_per_block,
+__global__ __launch_bounds__(256) void cg_pap_fix_kernel(int nchunks, int chunks_per_block,
                                                          const double *__restrict__ p, double *Ap,
-                                                         double *__restrict__ partials, int vec, int nchunks,
+                                                         const double *__restrict__ chunk_pap,
+                                                         double *__restrict__ partials,
                                                          const int *__restrict__ pos,
                                                          const int *__restrict__ chunk_row,
                                                          const double *__restrict__ part_first,
-                                                         const double *__restrict__ part_last,
-                                                         const int *__restrict__ block_c) {
+                                                         const double *__restrict__ part_last) {
   __shared__ double lds4[4];
-  const int c0 = block_c[blockIdx.x], c1 = block_c[blockIdx.x + 1];
-  for (int base = c0; base < c1; base += 256) {
-    const long long c = (long long)base + threadIdx.x;
-    rowsplit_complete_row<double, CH>(c < c1 ? c : nchunks, nchunks, pos, chunk_row, part_first, part_last, Ap, 0);
-  }
-  __syncthreads();
-  const long long r0 = std::min(n, (long long)blockIdx.x * rows_per_block);
-  const long long r1 = std::min(n, r0 + rows_per_block);
+  const long long c0 = (long long)blockIdx.x * chunks_per_block;
+  const long long c1 = std::min<long long>(nchunks, c0 + chunks_per_block);
   double acc = 0.0;
-  if (vec) {
-    for (long long i = r0 / 2 + threadIdx.x; i < r1 / 2; i += 256) {
-      const v2d a = ld2(p, i), b = ld2(Ap, i);
-      acc = acc + a.x * b.x;
-      acc = acc + a.y * b.y;
+  for (long long base = c0; base < c1; base += 256) {
+    const long long c = base + threadIdx.x;
+    const bool mine = c < c1;
+    bool owner;
+    int r;
+    const double total = rowsplit_row_total<double, CH>((mine && c >= 1) ? c : nchunks, nchunks, pos, chunk_row,
+                                                        part_first, part_last, owner, r);
+    if (owner) {
+      Ap[r] = total;
+      acc = acc + p[r] * total;
     }
-    if ((r1 & 1) && threadIdx.x == 0) acc = acc + p[r1 - 1] * Ap[r1 - 1];  // r1 is odd only where it is n
-  } else {
-    for (long long i = r0 + threadIdx.x; i < r1; i += 256) acc = acc + p[i] * Ap[i];
+    if (mine) acc = acc + chunk_pap[c];
   }
   const double bsum = block_sum_256d(acc, lds4);
   if (threadIdx.x == 0) partials[blockIdx.x] = bsum;
 }
 
-// block_c[b] = first chunk boundary c in [1, nchunks] whose row chunk_row[c] is at or behind
-// row b * rows_per_block (b = 0 .. blocks); chunk_row ascends and chunk_row[nchunks] is n.
-__global__ __launch_bounds__(256) void cg_fix_ranges_kernel(int blocks, long long n, long long rows_per_block,
-                                                            int nchunks, const int *__restrict__ chunk_row,
-                                                            int *__restrict__ block_c) {
-  const int b = blockIdx.x * 256 + threadIdx.x;
-  if (b > blocks) return;
-  const long long r = std::min(n, (long long)b * rows_per_block);
-  int lo = 1, hi = nchunks;
-  while (lo < hi) {
-    const int mid = lo + (hi - lo) / 2;
-    if (chunk_row[mid] >= r) hi = mid; else lo = mid + 1;
-  }
-  block_c[b] = lo;
-}
-
-// x += alpha p ; r -= alpha Ap ; block partials of r.r.   alpha = r.z / p.Ap with p.Ap
-// summed here from the partials the p.Ap kernel left.  x is touched once per iteration and Ap is read
-// here for the last time: both go through streaming accesses, so that they do not push p, which the next
-// SpMV gathers from, out of the caches (config 5: iteration 0.2615 -> 0.2510 ms, the SpMV kernel inside it
-// 0.147 -> 0.137 ms).
-__global__ __launch_bounds__(256) void cg_update_xr_kernel(long long n, const double *__restrict__ p,
-                                                           const double *__restrict__ Ap, double *__restrict__ x,
-                                                           double *__restrict__ r, CgState *st,
-                                                           unsigned long long iter, int count,
-                                                           const double *__restrict__ pap_partials,
-                                                           double *__restrict__ rr_partials, int vec) {
+// r -= alpha Ap ; block partials of r.r.   alpha = r.z / p.Ap with p.Ap summed here from the
+// partials the p.Ap kernel left; block 0 keeps alpha for the kernel that updates x and p.
+// Ap is read here for the last time: it goes through streaming accesses, so that it does not
+// push p, which the next SpMV gathers from, out of the caches.
+__global__ __launch_bounds__(256) void cg_update_r_kernel(long long n, const double *__restrict__ Ap,
+                                                          double *__restrict__ r, CgState *st,
+                                                          unsigned long long iter, int count,
+                                                          const double *__restrict__ pap_partials,
+                                                          double *__restrict__ rr_partials, int vec) {
   __shared__ double lds4[4];
-  if (block_sees_done(st)) return;
+  if (block_done_iter(st)) return;
   const double pAp = ordered_total(pap_partials, count, lds4);
   const double alpha = st->rz[iter & 1] / pAp;
   const double malpha = -alpha;
-  if (blockIdx.x == 0 && threadIdx.x == 0) st->pAp = pAp;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    st->pAp = pAp;
+    st->alpha = alpha;
+  }
   double rr = 0.0;
   const long long nv = vec ? n / 2 : 0;
   CG_GRID_STRIDE(i, 0, nv) {
-    const v2d pv = ld2(p, i), av = load_stream(reinterpret_cast<const v2d *>(Ap) + i);
-    v2d xv = load_stream(reinterpret_cast<const v2d *>(x) + i), rv = ld2(r, i);
-    xv.x = xv.x + pv.x * alpha;
-    xv.y = xv.y + pv.y * alpha;
+    const v2d av = load_stream(reinterpret_cast<const v2d *>(Ap) + i);
+    v2d rv = ld2(r, i);
     rv.x = rv.x + av.x * malpha;
     rv.y = rv.y + av.y * malpha;
-    store_stream(reinterpret_cast<v2d *>(x) + i, xv);
     st2(r, i, rv);
     rr = rr + rv.x * rv.x;
     rr = rr + rv.y * rv.y;
   }
   CG_GRID_STRIDE(i, 2 * nv, n) {
-    const double xt = p[i] * alpha;
-    const double xi = x[i] + xt;
     const double rt = Ap[i] * malpha;
     const double ri = r[i] + rt;
-    x[i] = xi;
     r[i] = ri;
     rr = rr + ri * ri;
   }
@@ -226,10 +207,7 @@ __device__ __forceinline__ bool cg_continues(CgState *st, unsigned long long ite
   if (blockIdx.x == 0 && threadIdx.x == 0) {
     st->rr = rr;
     st->relres = relres;
-    if (!go_on) {
-      st->iter = iter;
-      st->done = 1;
-    }
+    if (!go_on) st->done_iter = iter;
   }
   return go_on;
 }
@@ -241,7 +219,7 @@ __global__ __launch_bounds__(256) void cg_precond_kernel(long long n, const doub
                                                          const double *__restrict__ rr_partials,
                                                          double *__restrict__ rz_partials, int vec, int divide) {
   __shared__ double lds4[4];
-  if (block_sees_done(st)) return;
+  if (block_done_iter(st)) return;  // an earlier pass left, or block 0 of this kernel has just decided to
   const double rr = ordered_total(rr_partials, count, lds4);
   if (!cg_continues(st, iter, rr)) return;
   double acc = 0.0;
@@ -289,30 +267,56 @@ __global__ __launch_bounds__(256) void normalize_mom2_kernel(long long n, const 
   }
 }
 
-// p = z + beta p with beta = (new r.z) / (old r.z).  Unpreconditioned, z is r and the
-// new r.z is r.r: this kernel then makes the convergence test itself; preconditioned,
-// the test was made by cg_precond_kernel and `partials` holds r.z.
-__global__ __launch_bounds__(256) void cg_update_p_kernel(long long n, const double *__restrict__ z,
-                                                          double *__restrict__ p, CgState *st,
-                                                          unsigned long long iter, int count,
-                                                          const double *__restrict__ partials, int preconditioned,
-                                                          int vec) {
+// x += alpha p ; p = z + beta p with beta = (new r.z) / (old r.z).  Unpreconditioned, z is r
+// and the new r.z is r.r: this kernel then makes the convergence test itself; preconditioned,
+// the test was made by cg_precond_kernel and `partials` holds r.z.  The pass that leaves
+// (the exit mark names this very iteration) still owes x its alpha p and keeps p as it is;
+// passes queued behind it find an older mark and touch nothing.  x goes through streaming
+// accesses: it is touched once per iteration and must not push p out of the caches.
+__global__ __launch_bounds__(256) void cg_update_xp_kernel(long long n, const double *__restrict__ z,
+                                                           double *__restrict__ p, double *__restrict__ x,
+                                                           CgState *st, unsigned long long iter, int count,
+                                                           const double *__restrict__ partials, int preconditioned,
+                                                           int vec) {
   __shared__ double lds4[4];
-  if (block_sees_done(st)) return;
+  const unsigned long long mark = block_done_iter(st);
+  if (mark != 0 && mark != iter) return;
   const double rz_new = ordered_total(partials, count, lds4);
-  if (!preconditioned && !cg_continues(st, iter, rz_new)) return;
+  const bool go_on = preconditioned ? mark == 0 : cg_continues(st, iter, rz_new);
+  const double alpha = st->alpha;
+  const long long nv = vec ? n / 2 : 0;
+  if (!go_on) {
+    CG_GRID_STRIDE(i, 0, nv) {
+      const v2d pv = ld2(p, i);
+      v2d xv = load_stream(reinterpret_cast<const v2d *>(x) + i);
+      xv.x = xv.x + pv.x * alpha;
+      xv.y = xv.y + pv.y * alpha;
+      store_stream(reinterpret_cast<v2d *>(x) + i, xv);
+    }
+    CG_GRID_STRIDE(i, 2 * nv, n) {
+      const double xt = p[i] * alpha;
+      x[i] = x[i] + xt;
+    }
+    return;
+  }
   const double beta = rz_new / st->rz[iter & 1];
   if (blockIdx.x == 0 && threadIdx.x == 0) st->rz[(iter + 1) & 1] = rz_new;
-  const long long nv = vec ? n / 2 : 0;
   CG_GRID_STRIDE(i, 0, nv) {
     const v2d zv = load_stream(reinterpret_cast<const v2d *>(z) + i);
     v2d pv = ld2(p, i);
+    v2d xv = load_stream(reinterpret_cast<const v2d *>(x) + i);
+    xv.x = xv.x + pv.x * alpha;
+    xv.y = xv.y + pv.y * alpha;
+    store_stream(reinterpret_cast<v2d *>(x) + i, xv);
     pv.x = zv.x + pv.x * beta;
     pv.y = zv.y + pv.y * beta;
     st2(p, i, pv);
   }
   CG_GRID_STRIDE(i, 2 * nv, n) {
-    const double pt = p[i] * beta;
+    const double pi = p[i];
+    const double xt = pi * alpha;
+    x[i] = x[i] + xt;
+    const double pt = pi * beta;
     p[i] = z[i] + pt;
   }
 }
@@ -326,8 +330,7 @@ __global__ __launch_bounds__(256) void cg_init_scalar_kernel(int count, const do
   if (threadIdx.x == 0) {
     st->initres = sqrt(trr);
     st->rz[1] = trz;  // the first iteration is i = 1
-    st->iter = 1;
-    st->done = 0;
+    st->done_iter = 0;
   }
 }
 
@@ -362,6 +365,7 @@ int pcg_run(lapis_hip_csr_plan *plan, int64_t n, const int32_t *pos, const int32
   int64_t stride = n;  // distance between the four work vectors
   CgState *state = nullptr;
   double *partials = nullptr;
+  double *chunk_pap = nullptr;  // per chunk of the row-split SpMV: p.Ap over the rows inside it
   bool finished = false;
 
   // one-exit cleanup
@@ -370,6 +374,7 @@ int pcg_run(lapis_hip_csr_plan *plan, int64_t n, const int32_t *pos, const int32
     if (own_work) (void)hipFree(own_work);
     if (state) (void)hipFree(state);
     if (partials) (void)hipFree(partials);
+    if (chunk_pap) (void)hipFree(chunk_pap);
   };
 #define PCG_TRY(expr)                                                                          \
   do {                                                                                         \
@@ -408,7 +413,9 @@ int pcg_run(lapis_hip_csr_plan *plan, int64_t n, const int32_t *pos, const int32
   double *tmp = mask ? work + 4 * stride : nullptr;
   const int divide = mask ? 1 : 0;
   PCG_TRY(hipMalloc(&state, sizeof(CgState)));
-  PCG_TRY(hipMalloc(&partials, sizeof(double) * 3 * kDotMaxBlocks + sizeof(int) * (kDotMaxBlocks + 1)));
+  PCG_TRY(hipMalloc(&partials, sizeof(double) * 3 * kDotMaxBlocks));
+  if (!mask && plan->stats.kernel == LAPIS_HIP_SPMV_NNZSPLIT && plan->nchunks > 1)
+    PCG_TRY(hipMalloc(&chunk_pap, sizeof(double) * (size_t)plan->nchunks));
   CgState h{};
   h.maxiter = maxiter;
   h.tol = tol;
@@ -425,12 +432,7 @@ int pcg_run(lapis_hip_csr_plan *plan, int64_t n, const int32_t *pos, const int32
   hipLaunchKernelGGL(cg_init_scalar_kernel, dim3(1), dim3(256), 0, st, grid, partials, state);
   PCG_TRY(hipGetLastError());
   double *pap_partials = partials, *rr_partials = partials + kDotMaxBlocks, *rz_partials = partials + 2 * kDotMaxBlocks;
-  // rows per block of the p.Ap kernel that also completes the rows the row-split SpMV cuts (an even number)
-  int *block_c = reinterpret_cast<int *>(partials + 3 * kDotMaxBlocks);
-  const long long rows_per_block = ((((long long)n + grid - 1) / grid) + 1) & ~1LL;
-  bool ranges_ready = false;
-
-  // The host looks at the device's `done` flag after each batch of iterations; a
+  // The host looks at the device's exit mark after each batch of iterations; a
   // batch queued past convergence costs launches only (its kernels return at once
   // or touch scratch vectors only).
   uint64_t launched = 0;
@@ -453,19 +455,20 @@ int pcg_run(lapis_hip_csr_plan *plan, int64_t n, const int32_t *pos, const int32
         hipLaunchKernelGGL(masked_combine_kernel, dim3(grid), dim3(256), 0, st, (long long)n, 0, dinv, tmp, mask, Ap);
       } else {
         // Ap = A p: the reference zero-fills Ap and accumulates (examples/pcg_solve.py:12-19)
-        PCG_RC(spmv_overwrite_f64(plan, n, n, pos, crd, val, p, Ap, stream, &deferred));
+        PCG_RC(spmv_overwrite_f64(plan, n, n, pos, crd, val, p, Ap, stream, chunk_pap ? &deferred : nullptr,
+                                  chunk_pap));
       }
       const unsigned long long iter = launched + (uint64_t)it + 1;  // the reference's counter for this pass
+      int pap_count = grid;
       if (deferred) {
-        if (!ranges_ready) {
-          hipLaunchKernelGGL(cg_fix_ranges_kernel, dim3((grid + 256) / 256), dim3(256), 0, st, grid, (long long)n,
-                             rows_per_block, plan->nchunks, (const int *)plan->chunk_row, block_c);
-          ranges_ready = true;
-        }
-#define PCG_PAP_FIX(CH)                                                                                              \
-  hipLaunchKernelGGL(cg_pap_fix_kernel<CH>, dim3(grid), dim3(256), 0, st, (long long)n, rows_per_block, p, Ap,       \
-                     pap_partials, vec, plan->nchunks, pos, (const int *)plan->chunk_row,                            \
-                     (const double *)plan->part_first, (const double *)plan->part_last, (const int *)block_c)
+        // one thread per chunk, at most kDotMaxBlocks blocks
+        const int nchunks = plan->nchunks;
+        const int per_block = (int)std::max<int64_t>(256, ceil_div(ceil_div(nchunks, kDotMaxBlocks), 256) * 256);
+        pap_count = (int)ceil_div(nchunks, per_block);
+#define PCG_PAP_FIX(CH)                                                                                         \
+  hipLaunchKernelGGL(cg_pap_fix_kernel<CH>, dim3(pap_count), dim3(256), 0, st, nchunks, per_block, p, Ap,        \
+                     (const double *)chunk_pap, pap_partials, pos, (const int *)plan->chunk_row,                \
+                     (const double *)plan->part_first, (const double *)plan->part_last)
         switch (deferred) {
           case 512: PCG_PAP_FIX(512); break;
           case 1024: PCG_PAP_FIX(1024); break;
@@ -478,21 +481,21 @@ int pcg_run(lapis_hip_csr_plan *plan, int64_t n, const int32_t *pos, const int32
       } else {
         hipLaunchKernelGGL(cg_pap_kernel, dim3(grid), dim3(256), 0, st, (long long)n, p, Ap, pap_partials, vec);
       }
-      hipLaunchKernelGGL(cg_update_xr_kernel, dim3(grid), dim3(256), 0, st, (long long)n, p, Ap, x, r, state, iter,
-                         grid, pap_partials, rr_partials, vec);
+      hipLaunchKernelGGL(cg_update_r_kernel, dim3(grid), dim3(256), 0, st, (long long)n, Ap, r, state, iter,
+                         pap_count, pap_partials, rr_partials, vec);
       if (pre)
         hipLaunchKernelGGL(cg_precond_kernel, dim3(grid), dim3(256), 0, st, (long long)n, r, dinv, z, state, iter,
                            grid, rr_partials, rz_partials, vec, divide);
-      hipLaunchKernelGGL(cg_update_p_kernel, dim3(grid), dim3(256), 0, st, (long long)n, z, p, state, iter, grid,
-                         pre ? rz_partials : rr_partials, pre, vec);
+      hipLaunchKernelGGL(cg_update_xp_kernel, dim3(grid), dim3(256), 0, st, (long long)n, z, p, x, state, iter,
+                         grid, pre ? rz_partials : rr_partials, pre, vec);
       PCG_TRY(hipGetLastError());
     }
     launched += (uint64_t)todo;
     CgState now;
     PCG_TRY(hipMemcpyAsync(&now, state, sizeof(now), hipMemcpyDeviceToHost, st));
     PCG_TRY(hipStreamSynchronize(st));
-    if (now.done) {
-      *iters = now.iter;
+    if (now.done_iter != 0) {
+      *iters = now.done_iter;
       *relres = now.relres;
       finished = true;
     }

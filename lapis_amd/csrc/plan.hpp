@@ -84,8 +84,10 @@ template <typename T>
 int gather_values(const unsigned *perm, const T *val, T *out, int64_t nnz, hipStream_t st);
 
 // y = A x without reading y; defined in spmv.hip.  A caller that passes `deferred_chunk` and gets a
-// non-zero chunk length back completes the rows cut at chunk boundaries itself (rowsplit_fix.hpp).
+// non-zero chunk length back completes the rows cut at chunk boundaries itself (rowsplit_fix.hpp);
+// for a square matrix `xy_chunk` (plan->nchunks doubles) then holds, per chunk, the sum of
+// x[r]*y[r] over the rows that lie wholly inside the chunk.
 int spmv_overwrite_f64(lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, const int32_t *pos,
                        const int32_t *crd, const double *val, const double *x, double *y,
-                       lapis_hip_stream_t stream, int *deferred_chunk = nullptr);
+                       lapis_hip_stream_t stream, int *deferred_chunk = nullptr, double *xy_chunk = nullptr);
 }  // namespace lapis

@@ -9,19 +9,21 @@
 namespace lapis {
 
 // Called by ALL 64 lanes of a wavefront, lane l for chunk boundary c (1 <= c; lanes
-// with c >= nchunks take part and do nothing).  The row cut by boundary c is
-// completed by the lane of the FIRST boundary that cuts it:
-//   y[r] (+)= part_last[c-1] + part_first[c] + ... + part_first[c_last]
-// in that fixed order, so the result does not depend on scheduling.  Rows cut 16
+// with c >= nchunks take part and own nothing).  The row cut by boundary c belongs
+// to the lane of the FIRST boundary that cuts it; for that lane `owner` is set, `r`
+// is the row and the value returned is
+//   part_last[c-1] + part_first[c] + ... + part_first[c_last]
+// summed in that fixed order, so the result does not depend on scheduling.  Rows cut 16
 // times or more are summed by the whole wavefront.
 template <typename T, int CH>
-__device__ __forceinline__ void rowsplit_complete_row(long long c, int nchunks, const int *__restrict__ pos,
-                                                      const int *__restrict__ chunk_row,
-                                                      const T *__restrict__ part_first,
-                                                      const T *__restrict__ part_last, T *y, int accumulate) {
+__device__ __forceinline__ T rowsplit_row_total(long long c, int nchunks, const int *__restrict__ pos,
+                                                const int *__restrict__ chunk_row,
+                                                const T *__restrict__ part_first,
+                                                const T *__restrict__ part_last, bool &owner, int &r) {
   const int lane = threadIdx.x & 63;
-  bool owner = false;
-  int r = 0, cfirst = 0, clast = -1;
+  owner = false;
+  r = 0;
+  int cfirst = 0, clast = -1;
   if (c < nchunks) {
     r = chunk_row[c];
     const long long ps = pos[r];
@@ -49,6 +51,18 @@ __device__ __forceinline__ void rowsplit_complete_row(long long c, int nchunks, 
     part = group_sum<64>(part);
     if (lane == src) total = part_last[cfirst - 1] + part;
   }
+  return total;
+}
+
+// The same call convention; the owner writes y[r] (+)= the row's total.
+template <typename T, int CH>
+__device__ __forceinline__ void rowsplit_complete_row(long long c, int nchunks, const int *__restrict__ pos,
+                                                      const int *__restrict__ chunk_row,
+                                                      const T *__restrict__ part_first,
+                                                      const T *__restrict__ part_last, T *y, int accumulate) {
+  bool owner;
+  int r;
+  const T total = rowsplit_row_total<T, CH>(c, nchunks, pos, chunk_row, part_first, part_last, owner, r);
   if (owner) y[r] = accumulate ? total + y[r] : total;
 }
 

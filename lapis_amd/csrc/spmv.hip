@@ -204,12 +204,15 @@ __global__ __launch_bounds__(64 * WAVES) void spmv_rowblock_kernel(
 // A row piece that is a whole row is written to y at once; a piece of a row that
 // started in an earlier chunk goes to part_first[c], a piece of a row that
 // continues into the next chunk to part_last[c]; the fix-up kernel adds them up.
+// With `xy_chunk` (square matrices) the wavefront also leaves xy_chunk[c] = sum of
+// x[r] * (A x)[r] over the rows r that lie wholly inside its chunk, lanes summed in a
+// fixed order: the p.Ap of a CG iteration without a second pass over the vectors.
 template <typename T, int CH, int WAVES, bool VEC, bool NT>
 __global__ __launch_bounds__(64 * WAVES) void spmv_nnzsplit_kernel(
     int nrows, int nnz, int nchunks, const int *__restrict__ pos, const int *__restrict__ crd,
     const T *__restrict__ val, const T *__restrict__ x, T *__restrict__ y,
     const int *__restrict__ chunk_row, T *__restrict__ part_first, T *__restrict__ part_last, int accumulate,
-    int xcd_map) {
+    int xcd_map, double *__restrict__ xy_chunk) {
   __shared__ T lds[WAVES * CH];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -226,12 +229,15 @@ __global__ __launch_bounds__(64 * WAVES) void spmv_nnzsplit_kernel(
   stage_products<T, CH, VEC, NT>(buf, lane, crd, val, x, e0, len, len);
   wave_lds_sync();
 
+  double xy = 0.0;
   for (long long rb = r0; rb <= r1;) {
     const long long r = rb + lane;
     int ps = 0, pe = 0;
+    T xr = T(0);  // asked for together with the positions, so that its latency hides behind the row sums
     if (r <= r1) {
       ps = ld<NT>(pos + r);
       pe = ld<NT>(pos + r + 1);
+      if (xy_chunk) xr = x[r];
     }
     const int lo = std::max(ps, e0) - e0;
     const int hi = (int)(std::min<long long>(pe, e1) - e0);
@@ -239,9 +245,10 @@ __global__ __launch_bounds__(64 * WAVES) void spmv_nnzsplit_kernel(
     if (hi > lo) {
       const bool starts = ps >= e0;
       const bool ends = pe <= e1;
-      if (starts && ends)
+      if (starts && ends) {
         y[r] = accumulate ? acc + y[r] : acc;
-      else if (!starts)
+        xy = xy + (double)xr * (double)acc;
+      } else if (!starts)
         part_first[c] = acc;
       else
         part_last[c] = acc;
@@ -262,6 +269,10 @@ __global__ __launch_bounds__(64 * WAVES) void spmv_nnzsplit_kernel(
       next = lo_r;
     }
     rb = next;
+  }
+  if (xy_chunk) {
+    xy = group_sum<64>(xy);
+    if (lane == 0) xy_chunk[c] = xy;
   }
 }
 
@@ -500,13 +511,13 @@ int launch_rowblock(int64_t nrows, int64_t nnz, const int *pos, const int *crd, 
 
 template <typename T, bool VEC, bool NT, int CH, int WPB>
 int launch_nnzsplit_cfg(const lapis_hip_csr_plan *p, const int *pos, const int *crd, const T *val, const T *x,
-                        T *y, hipStream_t st, int accumulate, bool defer_fixup) {
+                        T *y, hipStream_t st, int accumulate, bool defer_fixup, double *xy_chunk) {
   const int nchunks = p->nchunks;
   const int blocks = (int)ceil_div(nchunks, WPB);
   launch_timed(spmv_nnzsplit_kernel<T, CH, WPB, VEC, NT>, dim3(blocks), dim3(64 * WPB),
                st, (int)p->stats.nrows, (int)p->stats.nnz, nchunks, pos, crd, val, x, y,
                (const int *)p->chunk_row, static_cast<T *>(p->part_first), static_cast<T *>(p->part_last), accumulate,
-               p->xcd_map);
+               p->xcd_map, xy_chunk);
   LAPIS_LAUNCH_CHECK();
   if (nchunks > 1 && !defer_fixup) {
     const int fblocks = (int)ceil_div(nchunks - 1, 256);
@@ -520,15 +531,16 @@ int launch_nnzsplit_cfg(const lapis_hip_csr_plan *p, const int *pos, const int *
 
 template <typename T, bool VEC, bool NT>
 int launch_nnzsplit(const lapis_hip_csr_plan *p, const int *pos, const int *crd, const T *val, const T *x,
-                    T *y, hipStream_t st, int accumulate = 1, bool defer_fixup = false) {
+                    T *y, hipStream_t st, int accumulate = 1, bool defer_fixup = false,
+                    double *xy_chunk = nullptr) {
   switch (p->stats.chunk * 16 + p->waves_per_block) {
-    case 512 * 16 + 4: return launch_nnzsplit_cfg<T, VEC, NT, 512, 4>(p, pos, crd, val, x, y, st, accumulate, defer_fixup);
-    case 512 * 16 + 8: return launch_nnzsplit_cfg<T, VEC, NT, 512, 8>(p, pos, crd, val, x, y, st, accumulate, defer_fixup);
-    case 1024 * 16 + 2: return launch_nnzsplit_cfg<T, VEC, NT, 1024, 2>(p, pos, crd, val, x, y, st, accumulate, defer_fixup);
-    case 1024 * 16 + 4: return launch_nnzsplit_cfg<T, VEC, NT, 1024, 4>(p, pos, crd, val, x, y, st, accumulate, defer_fixup);
-    case 1024 * 16 + 8: return launch_nnzsplit_cfg<T, VEC, NT, 1024, 8>(p, pos, crd, val, x, y, st, accumulate, defer_fixup);
-    case 2048 * 16 + 2: return launch_nnzsplit_cfg<T, VEC, NT, 2048, 2>(p, pos, crd, val, x, y, st, accumulate, defer_fixup);
-    case 2048 * 16 + 4: return launch_nnzsplit_cfg<T, VEC, NT, 2048, 4>(p, pos, crd, val, x, y, st, accumulate, defer_fixup);
+    case 512 * 16 + 4: return launch_nnzsplit_cfg<T, VEC, NT, 512, 4>(p, pos, crd, val, x, y, st, accumulate, defer_fixup, xy_chunk);
+    case 512 * 16 + 8: return launch_nnzsplit_cfg<T, VEC, NT, 512, 8>(p, pos, crd, val, x, y, st, accumulate, defer_fixup, xy_chunk);
+    case 1024 * 16 + 2: return launch_nnzsplit_cfg<T, VEC, NT, 1024, 2>(p, pos, crd, val, x, y, st, accumulate, defer_fixup, xy_chunk);
+    case 1024 * 16 + 4: return launch_nnzsplit_cfg<T, VEC, NT, 1024, 4>(p, pos, crd, val, x, y, st, accumulate, defer_fixup, xy_chunk);
+    case 1024 * 16 + 8: return launch_nnzsplit_cfg<T, VEC, NT, 1024, 8>(p, pos, crd, val, x, y, st, accumulate, defer_fixup, xy_chunk);
+    case 2048 * 16 + 2: return launch_nnzsplit_cfg<T, VEC, NT, 2048, 2>(p, pos, crd, val, x, y, st, accumulate, defer_fixup, xy_chunk);
+    case 2048 * 16 + 4: return launch_nnzsplit_cfg<T, VEC, NT, 2048, 4>(p, pos, crd, val, x, y, st, accumulate, defer_fixup, xy_chunk);
     default:
       return set_error(LAPIS_HIP_ERR_INVALID_ARGUMENT, "spmv: no row-split kernel for %d non-zeros per wavefront, %d wavefronts per block",
                        p->stats.chunk, p->waves_per_block);
@@ -612,9 +624,12 @@ namespace lapis {
 // itself (rowsplit_complete_row over boundaries 1..nchunks-1 with the plan's chunk_row,
 // part_first and part_last, accumulate = 0): when the row-split kernel runs, its fix-up
 // launch is left out and *deferred_chunk is the chunk length, otherwise it is 0 and y is complete.
+// In that case, and only then, `xy_chunk` (plan->nchunks doubles, square matrices) receives per
+// chunk the sum of x[r]*y[r] over the rows that lie wholly inside the chunk; the rows the caller
+// completes are missing from it.
 int spmv_overwrite_f64(lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, const int32_t *pos,
                        const int32_t *crd, const double *val, const double *x, double *y,
-                       lapis_hip_stream_t stream, int *deferred_chunk) {
+                       lapis_hip_stream_t stream, int *deferred_chunk, double *xy_chunk) {
   if (deferred_chunk) *deferred_chunk = 0;
   if (plan && plan->stats.kernel == LAPIS_HIP_SPMV_NNZSPLIT && plan->stats.empty_rows == 0 && plan->stats.nnz > 0 &&
       plan->stats.nrows == nrows && plan->stats.ncols == ncols && plan->pos == pos && aligned16(crd) &&
@@ -622,8 +637,10 @@ int spmv_overwrite_f64(lapis_hip_csr_plan *plan, int64_t nrows, int64_t ncols, c
     LAPIS_CHECK_INIT();
     hipStream_t st = as_stream(stream);
     const bool defer = deferred_chunk && plan->nchunks > 1;
-    const int rc = plan->nontemporal ? launch_nnzsplit<double, true, true>(plan, pos, crd, val, x, y, st, 0, defer)
-                                     : launch_nnzsplit<double, true, false>(plan, pos, crd, val, x, y, st, 0, defer);
+    double *xy = (defer && nrows == ncols) ? xy_chunk : nullptr;
+    const int rc = plan->nontemporal
+                       ? launch_nnzsplit<double, true, true>(plan, pos, crd, val, x, y, st, 0, defer, xy)
+                       : launch_nnzsplit<double, true, false>(plan, pos, crd, val, x, y, st, 0, defer, xy);
     if (rc == LAPIS_HIP_OK && defer) *deferred_chunk = plan->stats.chunk;
     return rc;
   }
