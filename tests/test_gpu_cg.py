@@ -76,6 +76,36 @@ def test_convergence_stops_early_and_x_is_not_touched_afterwards(gpu, oracle):
     assert i1 == 1
 
 
+@pytest.mark.parametrize("preconditioned", [False, True])
+def test_odd_size_and_unaligned_buffers_take_the_elementwise_paths(gpu, oracle, preconditioned):
+    """An odd n with a caller's work buffer puts two of the four work vectors on addresses that are
+    not multiples of 16, and x starts one element into its allocation: the vector kernels
+    then walk element by element, and must give what the 128-bit paths give."""
+    A, b = gen.config5(scale=(15 / 192) ** 3)
+    n = A.nrows
+    assert n % 2 == 1
+    import scipy.sparse as sp
+    M = sp.csr_matrix((A.val, A.crd, A.pos), shape=(n, n))
+    dinv = 1.0 / M.diagonal() if preconditioned else None
+    xo, io, ro = oracle.pcg(A.pos, A.crd, A.val, b, dinv if preconditioned else np.ones(n), 1e-9, 500)
+    dpos, dcrd = dev(A.pos), dev(A.crd)
+    plan = gpu.CsrPlan(n, n, dpos, dcrd)
+    xbuf = torch.full((n + 1,), 7.0, dtype=torch.float64, device="cuda")
+    x = xbuf[1:]
+    assert x.data_ptr() % 16 == 8
+    work = torch.empty(4 * n, dtype=torch.float64, device="cuda")
+    ig, rg = gpu.pcg(plan, n, dpos, dcrd, dev(A.val), dev(b), dev(dinv) if preconditioned else None, 1e-9, 500, x,
+                     work=work)
+    assert ig == io and rg <= 1e-9
+    assert np.allclose(x.cpu().numpy(), xo, rtol=1e-7, atol=1e-10)
+    assert float(xbuf[0]) == 7.0
+    # the aligned run of the same system
+    xa, ia, ra = _solve(gpu, A.pos, A.crd, A.val, b, dinv, 1e-9, 500)
+    assert ia == ig
+    assert np.allclose(x.cpu().numpy(), xa, rtol=1e-9, atol=1e-12)
+    assert abs(np.linalg.norm(b - M @ x.cpu().numpy()) / np.linalg.norm(b) - rg) < 1e-9
+
+
 def test_masked_cg_and_moments_match_oracle(gpu, oracle, golden):
     g = golden["hitting_times"]
     pos, crd, val, shape = read_mtx_csr("mht_A.mtx")
