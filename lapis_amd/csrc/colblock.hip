@@ -209,7 +209,7 @@ __global__ __launch_bounds__(256) void gather_values_kernel(long long n, const u
 }
 }  // namespace
 
-int sort_keys_with_perm(const unsigned long long *keys_in, int64_t nnz, int end_bit, unsigned long long **keys_out,
+int sort_keys_with_perm(const unsigned long long *keys_in, int64_t nnz, int begin_bit, int end_bit, unsigned long long **keys_out,
                         unsigned **perm, hipStream_t st) {
   unsigned *iota = nullptr;
   void *temp = nullptr;
@@ -231,11 +231,11 @@ int sort_keys_with_perm(const unsigned long long *keys_in, int64_t nnz, int end_
   if ((e = hipMalloc(perm, sizeof(unsigned) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
   hipLaunchKernelGGL(iota_kernel, dim3((unsigned)ceil_div(nnz, 256)), dim3(256), 0, st, (long long)nnz, iota);
   if ((e = hipGetLastError()) != hipSuccess) return fail(e, "index kernel");
-  if ((e = hipcub::DeviceRadixSort::SortPairs(nullptr, temp_bytes, keys_in, *keys_out, iota, *perm, (int)nnz, 0, end_bit,
+  if ((e = hipcub::DeviceRadixSort::SortPairs(nullptr, temp_bytes, keys_in, *keys_out, iota, *perm, (int)nnz, begin_bit, end_bit,
                                               st)) != hipSuccess)
     return fail(e, "radix sort sizing");
   if ((e = hipMalloc(&temp, temp_bytes ? temp_bytes : 1)) != hipSuccess) return fail(e, "hipMalloc");
-  if ((e = hipcub::DeviceRadixSort::SortPairs(temp, temp_bytes, keys_in, *keys_out, iota, *perm, (int)nnz, 0, end_bit,
+  if ((e = hipcub::DeviceRadixSort::SortPairs(temp, temp_bytes, keys_in, *keys_out, iota, *perm, (int)nnz, begin_bit, end_bit,
                                               st)) != hipSuccess)
     return fail(e, "radix sort");
   if ((e = hipStreamSynchronize(st)) != hipSuccess) return fail(e, "synchronize");
@@ -435,7 +435,7 @@ int build(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int slice_log
                      slice_log2, slice_bits, p->pos, crd, keys_in);
   if ((e = hipGetLastError()) != hipSuccess) return fail(e, "key kernel");
   {
-    const int rc = sort_keys_with_perm(keys_in, nnz, end_bit, &keys_out, &perm, st);
+    const int rc = sort_keys_with_perm(keys_in, nnz, 0, end_bit, &keys_out, &perm, st);
     if (rc != LAPIS_HIP_OK) {
       (void)hipFree(keys_in);
       (void)hipFree(val_out);

@@ -364,22 +364,28 @@ __global__ __launch_bounds__(256) void long_row_list_kernel(int nrows, const int
 // key = (block << (col_bits + row_bits)) | (column << row_bits) | row in block: sorted,
 // the entries of a block come slice by slice and by column inside a slice.  A long row
 // (flag set) belongs to block nblocks_nat + rank / rows, as row rank % rows.
-__global__ __launch_bounds__(256) void colgroup_keys_kernel(int nrows, int row_bits, int col_bits, int nblocks_nat,
-                                                            const int *__restrict__ long_flag,
+// One wavefront per 1024 consecutive entries; the row of an entry comes from the positions by
+// bisection between the rows of the chunk's first and last entry (lanes 0 and 1 find those), so
+// the cost does not depend on how the entries are spread over the rows.
+__global__ __launch_bounds__(256) void colgroup_keys_kernel(int nrows, long long nnz, int row_bits, int col_bits,
+                                                            int nblocks_nat, const int *__restrict__ long_flag,
                                                             const int *__restrict__ long_rank,
                                                             const int *__restrict__ pos,
                                                             const int *__restrict__ crd,
                                                             unsigned long long *__restrict__ keys) {
-  // one wavefront per row: coalesced over the row's entries
   const int lane = threadIdx.x & 63;
-  const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= nrows) return;
-  long long v = row;  // position in the blocked numbering
-  if (long_flag && long_flag[row]) v = ((long long)nblocks_nat << row_bits) + long_rank[row];
-  const unsigned long long rb = (unsigned long long)(v >> row_bits);
-  const unsigned long long rl = (unsigned long long)(v & ((1LL << row_bits) - 1));
-  const int s = pos[row], e = pos[row + 1];
-  for (int j = s + lane; j < e; j += 64) {
+  const long long j0 = ((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * 1024;
+  if (j0 >= nnz) return;
+  const long long j1 = std::min(nnz, j0 + 1024);
+  int edge = 0;
+  if (lane < 2) edge = row_of_entry(pos, lane == 0 ? j0 : j1 - 1, 0, nrows - 1);
+  const int r_lo = __shfl(edge, 0, 64), r_hi = __shfl(edge, 1, 64);
+  for (long long j = j0 + lane; j < j1; j += 64) {
+    const int row = row_of_entry(pos, j, r_lo, r_hi);
+    long long v = row;  // position in the blocked numbering
+    if (long_flag && long_flag[row]) v = ((long long)nblocks_nat << row_bits) + long_rank[row];
+    const unsigned long long rb = (unsigned long long)(v >> row_bits);
+    const unsigned long long rl = (unsigned long long)(v & ((1LL << row_bits) - 1));
     const unsigned long long c = (unsigned long long)(unsigned)crd[j];
     keys[j] = (rb << (col_bits + row_bits)) | (c << row_bits) | rl;
   }
@@ -650,7 +656,8 @@ int build_colgroup(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int 
                      nblocks, nslices, slice_log2);
   }
 
-  // 2. sort the entries by (block, column, row in block)
+  // 2. sort the entries by (block, column, row in block): the entries arrive by rows and the sort is
+  // stable, so the bits of the row in its block need no passes of their own
   const size_t ntiles = (size_t)nblocks * ((size_t)nslices + 1);
   if ((e = hipMalloc(&keys_in, sizeof(unsigned long long) * (size_t)nnz)) != hipSuccess) return fail(e, "hipMalloc");
   // kPcPad entries behind both arrays: the producer wavefronts load whole chunks
@@ -662,13 +669,13 @@ int build_colgroup(lapis_hip_csr_plan *p, const int32_t *crd, const T *val, int 
   if ((e = hipMemsetAsync(fault, 0, sizeof(int), st)) != hipSuccess) return fail(e, "hipMemsetAsync");
   if ((e = hipMalloc(&tile_ptr, sizeof(int) * ntiles)) != hipSuccess) return fail(e, "hipMalloc");
   if ((e = hipMalloc(&block_range, sizeof(int) * 2 * (size_t)nblocks)) != hipSuccess) return fail(e, "hipMalloc");
-  hipLaunchKernelGGL(colgroup_keys_kernel, dim3((unsigned)ceil_div(nrows, 4)), dim3(256), 0, st, (int)nrows, row_bits,
-                     col_bits, nblocks_nat, nlong > 0 ? (const int *)long_flag : (const int *)nullptr,
+  hipLaunchKernelGGL(colgroup_keys_kernel, dim3((unsigned)ceil_div(ceil_div(nnz, 1024), 4)), dim3(256), 0, st,
+                     (int)nrows, (long long)nnz, row_bits, col_bits, nblocks_nat, nlong > 0 ? (const int *)long_flag : (const int *)nullptr,
                      (const int *)long_rank, p->pos, crd, keys_in);
   if ((e = hipGetLastError()) != hipSuccess) return fail(e, "key kernel");
   // the permutation of the sort is kept: lapis_hip_csr_plan_update_values refreshes the copy's values with it
   {
-    const int rc = sort_keys_with_perm(keys_in, nnz, end_bit, &keys_out, &perm, st);
+    const int rc = sort_keys_with_perm(keys_in, nnz, row_bits, end_bit, &keys_out, &perm, st);
     if (rc != LAPIS_HIP_OK) {
       release(true);
       return rc;

@@ -84,6 +84,17 @@ __device__ __forceinline__ V ldv(const V *p) {
   return *p;
 }
 
+// Largest row r in [lo, hi] with pos[r] <= j: the row that holds non-zero j when the positions
+// ascend.  The structure has not been validated when this runs: whatever pos holds, the
+// search ends after log2(hi - lo) steps and stays inside [lo, hi].
+__device__ __forceinline__ int row_of_entry(const int *__restrict__ pos, long long j, int lo, int hi) {
+  while (lo < hi) {
+    const int mid = (int)(((long long)lo + hi + 1) >> 1);
+    if (pos[mid] <= j) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+
 // Row sums in LDS are doubles for every value type: ds_add_f32 runs at a tenth of the
 // rate of ds_add_f64 on this chip (203 against 1780 G adds/s over random words, measured).
 __device__ __forceinline__ void lds_add(double *p, double v) { unsafeAtomicAdd(p, v); }

@@ -77,7 +77,7 @@ void free_colblock(lapis_hip_csr_plan *plan);
 
 // Sorts `nnz` 64-bit keys (bits [0, end_bit)).  On success *keys_out holds the sorted keys and
 // *perm the position each sorted key had before (both device buffers, the caller frees them).
-int sort_keys_with_perm(const unsigned long long *keys_in, int64_t nnz, int end_bit, unsigned long long **keys_out,
+int sort_keys_with_perm(const unsigned long long *keys_in, int64_t nnz, int begin_bit, int end_bit, unsigned long long **keys_out,
                         unsigned **perm, hipStream_t st);
 // out[i] = val[perm[i]]
 template <typename T>

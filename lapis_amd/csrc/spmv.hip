@@ -299,9 +299,15 @@ struct DeviceStats {
   unsigned long long near[4];   // non-zeros with |column - row| <= 32, 64, 128, 256
 };
 
+// Every statistic is first reduced over the block and reaches the one DeviceStats with one
+// atomic per block and field: tens of thousands of atomics on the same few words would take
+// longer than reading the matrix.
 __global__ __launch_bounds__(256) void row_stats_kernel(int nrows, const int *__restrict__ pos,
                                                         DeviceStats *st) {
-  const int lane = threadIdx.x & 63;
+  __shared__ int s_mn[4], s_mx[4], s_bad[4];
+  __shared__ unsigned long long s_empt[4];
+  __shared__ double s_sq[4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int mn = INT32_MAX, mx = 0, bad = 0;
   unsigned long long empt = 0;
   double sq = 0.0;
@@ -322,6 +328,21 @@ __global__ __launch_bounds__(256) void row_stats_kernel(int nrows, const int *__
     sq += __shfl_xor(sq, o, 64);
   }
   if (lane == 0) {
+    s_mn[wave] = mn;
+    s_mx[wave] = mx;
+    s_bad[wave] = bad;
+    s_empt[wave] = empt;
+    s_sq[wave] = sq;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; ++w) {
+      mn = std::min(mn, s_mn[w]);
+      mx = std::max(mx, s_mx[w]);
+      bad |= s_bad[w];
+      empt += s_empt[w];
+      sq += s_sq[w];
+    }
     atomicMin(&st->min_len, mn);
     atomicMax(&st->max_len, mx);
     if (bad) atomicOr(&st->bad, 1);
@@ -330,65 +351,74 @@ __global__ __launch_bounds__(256) void row_stats_kernel(int nrows, const int *__
   }
 }
 
-// One wavefront per 1024 consecutive non-zeros: range check of the coordinates and
-// the column span (max - min) of the chunk, summed over chunks.  The mean span says
-// how much of x a wavefront's gathers wander over: small for stencils and bands,
-// the whole vector for uniformly random columns.
-__global__ __launch_bounds__(256) void crd_range_kernel(long long nnz, int ncols,
-                                                        const int *__restrict__ crd, DeviceStats *st) {
-  const int lane = threadIdx.x & 63;
-  const long long chunk = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
-  const long long j0 = chunk * 1024;
-  if (j0 >= nnz) return;
-  int mn = INT32_MAX, mx = INT32_MIN, bad = 0;
-  for (int k = lane; k < 1024 && j0 + k < nnz; k += 64) {
-    const int cj = crd[j0 + k];
-    if (cj < 0 || cj >= ncols) bad = 1;
-    mn = std::min(mn, cj);
-    mx = std::max(mx, cj);
-  }
-  for (int o = 32; o > 0; o >>= 1) {
-    mn = std::min(mn, __shfl_xor(mn, o, 64));
-    mx = std::max(mx, __shfl_xor(mx, o, 64));
-    bad |= __shfl_xor(bad, o, 64);
-  }
-  if (lane == 0) {
-    if (bad) atomicOr(&st->bad, 2);
-    atomicAdd(&st->span_sum, (unsigned long long)((long long)mx - (long long)mn));
-  }
-}
-
-// How much of the matrix lies in a band around the diagonal: one thread per row
-// (a plan-time pass; the reads are not coalesced), block totals added with one atomic each.
-__global__ __launch_bounds__(256) void band_stats_kernel(int nrows, long long nnz, const int *__restrict__ pos,
-                                                         const int *__restrict__ crd, DeviceStats *st) {
-  __shared__ unsigned long long tot[4];
-  if (threadIdx.x < 4) tot[threadIdx.x] = 0ull;
-  __syncthreads();
-  const long long r = (long long)blockIdx.x * 256 + threadIdx.x;
+// One wavefront per 1024 consecutive non-zeros, wavefronts striding over the chunks:
+//  * range check of the coordinates;
+//  * the column span (max - min) of the chunk, summed over chunks: the mean span says how
+//    much of x a wavefront's gathers wander over, small for stencils and bands, the whole
+//    vector for uniformly random columns;
+//  * how much of the matrix lies in a band around the diagonal (|column - row| <= 32 ... 256).
+// The row of an entry comes from the positions by bisection: lanes 0 and 1 find the rows of the
+// chunk's first and last entry, every lane then searches between those two.  The work is by
+// entries, so a row of a million entries costs what a million short rows cost.
+__global__ __launch_bounds__(256) void entry_stats_kernel(int nrows, long long nnz, int ncols,
+                                                          const int *__restrict__ pos,
+                                                          const int *__restrict__ crd, DeviceStats *st) {
+  __shared__ unsigned long long s_span[4], s_near[4][4];
+  __shared__ int s_bad[4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const long long nchunks = (nnz + 1023) / 1024;
   unsigned cnt[4] = {0u, 0u, 0u, 0u};
-  if (r < nrows) {
-    // the structure has not been validated yet: stay inside crd whatever pos holds, and spend nothing on a
-    // row whose positions decrease (the plan is refused for it anyway)
-    const long long first = std::max<long long>(0, pos[r]);
-    const long long last = pos[r + 1] < pos[r] ? first : std::min<long long>(nnz, pos[r + 1]);
-    for (long long j = first; j < last; ++j) {
-      const long long d = (long long)crd[j] - r;
+  unsigned long long span = 0ull;
+  int bad = 0;
+  for (long long chunk = (long long)blockIdx.x * 4 + wave; chunk < nchunks; chunk += (long long)gridDim.x * 4) {
+    const long long j0 = chunk * 1024;
+    const long long j1 = std::min(nnz, j0 + 1024);
+    int edge = 0;
+    if (lane < 2) edge = row_of_entry(pos, lane == 0 ? j0 : j1 - 1, 0, nrows - 1);
+    const int r_lo = __shfl(edge, 0, 64), r_hi = __shfl(edge, 1, 64);
+    int mn = INT32_MAX, mx = INT32_MIN;
+    for (long long j = j0 + lane; j < j1; j += 64) {
+      const int cj = crd[j];
+      if (cj < 0 || cj >= ncols) bad = 1;
+      mn = std::min(mn, cj);
+      mx = std::max(mx, cj);
+      const long long d = (long long)cj - row_of_entry(pos, j, r_lo, r_hi);
       const long long a = d < 0 ? -d : d;
       cnt[0] += a <= 32;
       cnt[1] += a <= 64;
       cnt[2] += a <= 128;
       cnt[3] += a <= 256;
     }
+    for (int o = 32; o > 0; o >>= 1) {
+      mn = std::min(mn, __shfl_xor(mn, o, 64));
+      mx = std::max(mx, __shfl_xor(mx, o, 64));
+    }
+    span += (unsigned long long)((long long)mx - (long long)mn);  // the same in every lane
   }
+  unsigned long long near[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    unsigned v = cnt[i];
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    if ((threadIdx.x & 63) == 0 && v) atomicAdd(&tot[i], (unsigned long long)v);
+    near[i] = cnt[i];
+    for (int o = 32; o > 0; o >>= 1) near[i] += __shfl_xor(near[i], o, 64);
+  }
+  for (int o = 32; o > 0; o >>= 1) bad |= __shfl_xor(bad, o, 64);
+  if (lane == 0) {
+    s_span[wave] = span;
+    s_bad[wave] = bad;
+    for (int i = 0; i < 4; ++i) s_near[wave][i] = near[i];
   }
   __syncthreads();
-  if (threadIdx.x < 4 && tot[threadIdx.x]) atomicAdd(&st->near[threadIdx.x], tot[threadIdx.x]);
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; ++w) {
+      span += s_span[w];
+      bad |= s_bad[w];
+      for (int i = 0; i < 4; ++i) near[i] += s_near[w][i];
+    }
+    if (bad) atomicOr(&st->bad, 2);
+    if (span) atomicAdd(&st->span_sum, span);
+    for (int i = 0; i < 4; ++i)
+      if (near[i]) atomicAdd(&st->near[i], near[i]);
+  }
 }
 
 template <int CH>
@@ -690,19 +720,14 @@ extern "C" int lapis_hip_csr_plan_create(lapis_hip_csr_plan **out, int64_t nrows
     LAPIS_HIP_TRY(hipMalloc(&dstats, sizeof(DeviceStats)));
     hipError_t e = hipMemcpyAsync(dstats, &init, sizeof(init), hipMemcpyHostToDevice, st);
     if (e == hipSuccess) {
-      const int blocks = (int)std::min<int64_t>(ceil_div(nrows, 256), 4096);
+      const int blocks = (int)std::min<int64_t>(ceil_div(nrows, 256), 1024);
       hipLaunchKernelGGL(row_stats_kernel, dim3(blocks), dim3(256), 0, st, (int)nrows, pos, dstats);
       e = hipGetLastError();
     }
     if (e == hipSuccess && crd && nnz > 0) {
-      const int blocks = (int)ceil_div(ceil_div(nnz, 1024), 4);
-      hipLaunchKernelGGL(crd_range_kernel, dim3(blocks), dim3(256), 0, st, (long long)nnz, (int)ncols, crd,
-                         dstats);
-      e = hipGetLastError();
-    }
-    if (e == hipSuccess && crd && nnz > 0) {
-      hipLaunchKernelGGL(band_stats_kernel, dim3((unsigned)ceil_div(nrows, 256)), dim3(256), 0, st, (int)nrows,
-                         (long long)nnz, pos, crd, dstats);
+      const int blocks = (int)std::min<int64_t>(ceil_div(ceil_div(nnz, 1024), 4), 2048);
+      hipLaunchKernelGGL(entry_stats_kernel, dim3(blocks), dim3(256), 0, st, (int)nrows, (long long)nnz, (int)ncols,
+                         pos, crd, dstats);
       e = hipGetLastError();
     }
     if (e == hipSuccess) e = hipMemcpyAsync(&host, dstats, sizeof(host), hipMemcpyDeviceToHost, st);
