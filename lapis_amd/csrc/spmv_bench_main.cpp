@@ -79,6 +79,22 @@ bool read_matrix_market(const std::string &path, Csr &A, std::string &err) {
     err = "bad size line";
     return false;
   }
+  if (m > INT32_MAX - 64 || n > INT32_MAX || entries > INT32_MAX) {
+    err = "sizes exceed the int32 index range";
+    return false;
+  }
+  // A header may claim anything: an entry takes at least four characters ("1 1\n"), so a
+  // count the rest of the file cannot hold is refused before memory is set aside for it.
+  {
+    const std::streamoff here = in.tellg();
+    in.seekg(0, std::ios::end);
+    const std::streamoff end = in.tellg();
+    in.seekg(here);
+    if (here < 0 || end < here || entries > (end - here) / 4 + 1) {
+      err = "file ends before all entries were read";
+      return false;
+    }
+  }
   struct Entry {
     int32_t r, c;
     double v;

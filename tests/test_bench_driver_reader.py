@@ -113,6 +113,11 @@ def test_reader_on_the_reference_matrices(name):
     ("%%MatrixMarket matrix coordinate real general\n2 2 2\n1 1 1.0\n3 1 2.0\n", "outside"),
     ("%%MatrixMarket matrix coordinate real general\n2 2 3\n1 1 1.0\n", "entries"),
     ("not a matrix market file\n", "header"),
+    # a header that claims more entries than the file can hold must not make the reader set memory aside for them
+    ("%%MatrixMarket matrix coordinate real symmetric\n4 4 42147483647\n1 1 2\n2 1 -1\n", "claimed entries"),
+    ("%%MatrixMarket matrix coordinate pattern general\n3 3 2000000000\n1 2\n2 3\n3 1\n", "claimed entries"),
+    ("%%MatrixMarket matrix coordinate real general\n4294967296 4 1\n1 1 1.0\n", "int32 rows"),
+    ("%%MatrixMarket matrix coordinate real general\n4 4294967296 1\n1 1 1.0\n", "int32 columns"),
 ])
 def test_reader_refuses_what_it_cannot_represent(tmp_path, text, why):
     path = tmp_path / "bad.mtx"
