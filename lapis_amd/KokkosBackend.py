@@ -165,7 +165,16 @@ class KokkosBackend:
         """{method name: entry point of the prebuilt module} for the module's public functions.
 
         The method name is the function's own (``main`` becomes ``lapis_main`` as in the emitter,
-        TranslateToKokkosCpp.cpp:2351-2355); the entry point is found by what the function computes."""
+        TranslateToKokkosCpp.cpp:2351-2355); the entry point is found by what the function computes.
+        Text that cannot be read as MLIR fails like any other module the reference cannot lower
+        (python/lapis/KokkosBackend.py:36), whatever the reader stumbled over."""
+        try:
+            return self._bind(moduleText)
+        except (_mt.ParseError, ValueError, IndexError, KeyError, AttributeError, RecursionError) as e:
+            raise Exception(_LOWERING_FAILED + "\nthe module text could not be read: %s%s" % (
+                "" if isinstance(e, _mt.ParseError) else type(e).__name__ + ": ", e))
+
+    def _bind(self, moduleText):
         try:
             c = _mt.Canonicalizer(moduleText)
             public = c.public()

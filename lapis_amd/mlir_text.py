@@ -29,7 +29,10 @@ def _match(text, i):
     while j < n and stack:
         ch = text[j]
         if ch == '"':
-            j = text.index('"', j + 1) + 1
+            k = text.find('"', j + 1)
+            if k < 0:
+                raise ParseError("a string that does not end: %r" % text[j:j + 30])
+            j = k + 1
             continue
         if ch in ">" and j > 0 and text[j - 1] == "-":
             j += 1

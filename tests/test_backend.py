@@ -136,3 +136,21 @@ def test_functions_in_the_vocabulary_bind_operation_by_operation():
     for text in (loop_nests.elementwise(loop_nests.CUBE_BODY), loop_nests.DOT_PRODUCT_REDUCTION):
         with pytest.raises(Exception, match=r"Lowering to Kokkos dialect failed[\s\S]*depth 1"):
             b.bind(text)
+
+
+@pytest.mark.parametrize("damage", [
+    lambda t: t[:len(t) // 2],                                     # cut off in the middle of a function
+    lambda t: t.replace("(", "", 1),                               # a bracket that never opens
+    lambda t: t.replace("func.func", 'func.func "', 1),            # a string that never ends
+    lambda t: t.replace("tensor<?xf64>", "tensor<?xf64", 1),       # a type that never closes
+    lambda t: t.replace(" = ", " = = ", 1),
+    lambda t: "",
+])
+@pytest.mark.parametrize("text", [M.SPMV, M.PCG, loop_nests.SPMV_INDEX])
+def test_text_that_is_not_mlir_fails_like_a_module_the_reference_cannot_lower(text, damage):
+    """python/lapis/KokkosBackend.py:36: whatever goes wrong before the Kokkos dialect is reached is
+    reported as one Exception with one text; the reader's own errors do not leak through."""
+    try:
+        KokkosBackend(decompose_tensors=True).bind(damage(text))
+    except Exception as e:
+        assert type(e) is Exception and str(e).startswith("Lowering to Kokkos dialect failed."), repr(e)
