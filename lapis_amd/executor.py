@@ -75,6 +75,12 @@ class Csr:
     def __init__(self, pos, crd, val, nrows, ncols):
         self.pos, self.crd, self.val, self.nrows, self.ncols = pos, crd, val, int(nrows), int(ncols)
         self.nnz = int(crd.shape[0])
+        # the kernels index with what the buffers hold: sizes that do not agree must stop here, on the host
+        if self.nrows < 0 or self.ncols < 0 or int(pos.shape[0]) != self.nrows + 1:
+            raise ValueError("a %d x %d CSR operand needs %d positions, got %d" % (
+                self.nrows, self.ncols, self.nrows + 1, int(pos.shape[0])))
+        if int(val.shape[0]) != self.nnz:
+            raise ValueError("a CSR operand with %d coordinates and %d values" % (self.nnz, int(val.shape[0])))
         self.plan = None
         self.products = 0
 
@@ -89,6 +95,13 @@ class Cell:
 
     def __init__(self, value=0.0):
         self.value = value
+
+
+def _same_size(what, *tensors):
+    """The kernels take one element count for all their operands: refuse, on the host, operands that differ."""
+    sizes = [int(t.numel()) for t in tensors]
+    if len(set(sizes)) > 1:
+        raise ValueError("%s over operands of %s elements" % (what, ", ".join(map(str, sizes))))
 
 
 def _elem(ty):
@@ -493,6 +506,13 @@ class Executor:
 
     def _csr_product(self, A, x, y, k=None):
         hip = self.hip
+        if k is None:
+            if x.numel() != A.ncols or y.numel() != A.nrows:
+                raise ValueError("a %d x %d matrix times a vector of %d elements into one of %d" % (
+                    A.nrows, A.ncols, x.numel(), y.numel()))
+        elif tuple(x.shape) != (A.ncols, k) or tuple(y.shape) != (A.nrows, k):
+            raise ValueError("a %d x %d matrix times a %s matrix into a %s one" % (
+                A.nrows, A.ncols, "x".join(map(str, x.shape)), "x".join(map(str, y.shape))))
         if A.plan is None:
             A.plan = hip.CsrPlan(A.nrows, A.ncols, A.pos, A.crd, value_bytes=A.val.element_size(), nnz=A.nnz)
         A.products += 1
@@ -511,6 +531,7 @@ class Executor:
         dtype = numpy.float32 if f32 else float
         ev = lambda expr: float(_ew.evaluate(expr, scalars, dtype))
         kind = call[0]
+        _same_size("an elementwise operation", dst, *operands)
         if kind == "fill":
             hip.fill(dst, ev(call[1]))
         elif kind == "copy":
@@ -621,10 +642,12 @@ class Executor:
                 return [in_vals[0]]
             d = dest(False)
             if d.data_ptr() != in_vals[0].data_ptr():
+                _same_size("linalg.copy", in_vals[0], d)
                 hip.copy(flat(in_vals[0]), flat(d))
             return give(d)
         if op == "linalg.dot":
             init = out_v.value if isinstance(out_v, Cell) else out_v
+            _same_size("linalg.dot", in_vals[0], in_vals[1])
             r = hip.dot_host(flat(in_vals[0]), flat(in_vals[1]), float(init))
             r = numpy.float32(r) if in_vals[0].element_size() == 4 else r
             if isinstance(out_v, Cell):
@@ -644,6 +667,7 @@ class Executor:
             spec = _LINALG_NAMED[op]
             d = dest(False)
             a, b = flat(in_vals[0]), flat(in_vals[1])
+            _same_size(op, a, b, d)
             if spec[0] == "axpby":
                 hip.axpby(spec[1], a, spec[2], b, flat(d))
             elif spec[0] == "mult":
@@ -681,6 +705,9 @@ class Executor:
             return None
         d = n.depth1
         count = self._val(env, d["n"]) if d["n"] in env else int(d["n"])
+        if count < 0 or any(int(self._val(env, a).shape[0]) < count
+                            for a in ([d["x"], d["y"]] if d["kind"] == "dot" else list(d["arrays"]) + [d["dst"]])):
+            raise ValueError("a loop over %d elements of a shorter buffer" % count)
         if d["kind"] == "dot":
             x, y = self._val(env, d["x"])[:count], self._val(env, d["y"])[:count]
             r = hip.dot_host(x, y, float(self._val(env, d["init"])))

@@ -187,3 +187,29 @@ def test_scalar_arithmetic_follows_the_types():
     t, c, k, r = e.run("scalars", [a, b, 7])
     assert isinstance(t, np.float32) and t == np.float32(a * b) + a and c == bool(t > b) and k == 20
     assert r == float(np.sqrt(np.float64(t)))
+
+
+def test_operands_whose_sizes_do_not_agree_stop_on_the_host():
+    """The kernels take pointers and one element count: a vector that is too short would be read past its end
+    on the device, so every size is compared before a call is made."""
+    A = spd(30, 7)
+    good = csr(A)
+    # positions that do not fit the declared number of rows, values that do not fit the coordinates
+    with pytest.raises(ValueError, match="positions"):
+        ex.Csr(good.pos[:-1], good.crd, good.val, 30, 30)
+    with pytest.raises(ValueError, match="values"):
+        ex.Csr(good.pos, good.crd, good.val[:-1], 30, 30)
+    # x shorter than the matrix has columns; z shorter than the product
+    e = make(M.SPMV_THEN_AXPBY)
+    with pytest.raises(ValueError, match="30 x 30 matrix times a vector of 29"):
+        e.run("residual", [csr(A), vec(np.ones(29)), vec(np.ones(30)), 1.0, 1.0])
+    assert "spmv" not in fake_hip.calls
+    e = make(M.SPMV_THEN_AXPBY)
+    with pytest.raises(ValueError, match="elementwise"):
+        e.run("residual", [csr(A), vec(np.ones(30)), vec(np.ones(12)), 1.0, 1.0])
+    assert "axpby" not in fake_hip.calls
+    # loop-level: a dot over the eight elements of u against a v that holds five
+    e = make(loop_nests.DOT)
+    with pytest.raises(ValueError, match="shorter buffer"):
+        e.run("inner", [vec(np.ones(8)), vec(np.ones(5)), 0.0])
+    assert "dot_host" not in fake_hip.calls and "dot" not in fake_hip.calls
