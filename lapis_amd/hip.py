@@ -275,8 +275,36 @@ def _suffix(t):
     raise TypeError("values must be float32 or float64, got %s" % t.dtype)
 
 
+def _holds(what, n, *tensors, like=None):
+    """The C ABI takes pointers and counts: a tensor with fewer than ``n`` elements, of another element type
+    than ``like`` or with gaps between its elements would be read or written past its end on the device, so it
+    is refused here.  Raw addresses (ints) and None pass: the caller vouches for them."""
+    for t in tensors:
+        if t is None or isinstance(t, int):
+            continue
+        if t.numel() < n:
+            raise ValueError("%s: an operand of %d elements where %d are needed" % (what, t.numel(), n))
+        if like is not None and not isinstance(like, int) and t.dtype != like.dtype:
+            raise TypeError("%s: operands of %s and %s" % (what, t.dtype, like.dtype))
+        if not t.is_contiguous():
+            raise ValueError("%s: an operand that is not contiguous" % what)
+
+
+def _indices(what, *tensors):
+    import torch
+    for t in tensors:
+        if t is not None and not isinstance(t, int) and t.dtype != torch.int32:
+            raise TypeError("%s: positions and coordinates are int32, got %s" % (what, t.dtype))
+
+
 def spmv(plan, nrows, ncols, pos, crd, val, x, y, stream=None):
     """y += A x.  ``plan`` may be None: the launch then follows the reference's own rule."""
+    _indices("spmv", pos, crd)
+    _holds("spmv", nrows + 1, pos)
+    _holds("spmv", ncols, x, like=val)
+    _holds("spmv", nrows, y, like=val)
+    if not isinstance(crd, int) and not isinstance(val, int) and crd is not None and val is not None:
+        _holds("spmv", crd.numel(), val)
     lib = init()
     fn = getattr(lib, "lapis_hip_spmv_csr_%s_i32" % _suffix(val))
     check(fn(plan.handle if plan is not None else None, nrows, ncols, _ptr(pos), _ptr(crd), _ptr(val), _ptr(x),
@@ -286,8 +314,15 @@ def spmv(plan, nrows, ncols, pos, crd, val, x, y, stream=None):
 
 def spmm(nrows, ncols, pos, crd, val, B, C, stream=None, plan=None):
     """C += A B with row-major B (ncols x k) and C (nrows x k); with a plan its statistics pick the kernel."""
-    lib = init()
     k = int(C.shape[1])
+    _indices("spmm", pos, crd)
+    _holds("spmm", nrows + 1, pos)
+    _holds("spmm", crd.numel(), val)
+    if B.dim() != 2 or C.dim() != 2 or int(B.shape[1]) != k or B.shape[0] < ncols or C.shape[0] < nrows or \
+            B.stride(1) != 1 or C.stride(1) != 1 or B.dtype != val.dtype or C.dtype != val.dtype:
+        raise ValueError("spmm: a %d x %d matrix of %s times B %s into C %s" % (
+            nrows, ncols, val.dtype, tuple(B.shape), tuple(C.shape)))
+    lib = init()
     if plan is not None:
         fn = getattr(lib, "lapis_hip_spmm_csr_%s_i32_plan" % _suffix(val))
         check(fn(plan.handle, nrows, ncols, k, _ptr(pos), _ptr(crd), _ptr(val), _ptr(B), int(B.stride(0)), _ptr(C),
@@ -306,6 +341,8 @@ def spmm_last_kernel():
 
 def dot(x, y, result, init_value=0.0, stream=None):
     """result[0] = init + x.y, with ``result`` a one-element device tensor (no host sync)."""
+    _holds("dot", int(x.shape[0]), x, y, like=x)
+    _holds("dot", 1, result, like=x)
     lib = init()
     fn = getattr(lib, "lapis_hip_dot_%s" % _suffix(x))
     check(fn(int(x.shape[0]), _ptr(x), _ptr(y), init_value, _ptr(result), _stream(stream)))
@@ -342,6 +379,7 @@ def calibrate_mix(mode, x, window_bytes, stream_buf, stream_bytes, gathers, cu_c
 
 def dot_host(x, y, init_value=0.0, stream=None):
     """init + x . y as a Python float: the entry point that returns the scalar to the host (blocking)."""
+    _holds("dot", int(x.shape[0]), x, y, like=x)
     lib = init()
     out = (_dbl if x.element_size() == 8 else _flt)(0.0)
     fn = getattr(lib, "lapis_hip_dot_%s_host" % _suffix(x))
@@ -351,6 +389,8 @@ def dot_host(x, y, init_value=0.0, stream=None):
 
 def axpby_dot(a, x, b, y, dst, z, result, init_value=0.0, stream=None):
     """dst = a*x + b*y and result = init + dst . z (z None: dst . dst) in one pass."""
+    _holds("axpby_dot", int(x.shape[0]), x, y, dst, z, like=x)
+    _holds("axpby_dot", 1, result, like=x)
     lib = init()
     fn = getattr(lib, "lapis_hip_axpby_dot_%s" % _suffix(x))
     check(fn(int(x.shape[0]), a, _ptr(x), b, _ptr(y), _ptr(dst), _ptr(z) if z is not None else None, init_value,
@@ -360,12 +400,15 @@ def axpby_dot(a, x, b, y, dst, z, result, init_value=0.0, stream=None):
 
 def dot_noalloc(x, y, result, init_value=0.0, stream=None):
     """dot() through the entry point that allocates nothing (fp64; fixed scratch inside the library)."""
+    _holds("dot_noalloc", int(x.shape[0]), x, y, like=x)
+    _holds("dot_noalloc", 1, result, like=x)
     lib = init()
     check(lib.lapis_hip_dot_f64_noalloc(int(x.shape[0]), _ptr(x), _ptr(y), init_value, _ptr(result), _stream(stream)))
     return result
 
 
 def axpby(a, x, b, y, dst, stream=None):
+    _holds("axpby", int(x.shape[0]), x, y, dst, like=x)
     lib = init()
     fn = getattr(lib, "lapis_hip_axpby_%s" % _suffix(x))
     check(fn(int(x.shape[0]), a, _ptr(x), b, _ptr(y), _ptr(dst), _stream(stream)))
@@ -373,11 +416,13 @@ def axpby(a, x, b, y, dst, stream=None):
 
 
 def mult(x, y, dst, stream=None):
+    _holds("mult", int(x.shape[0]), x, y, dst, like=x)
     check(getattr(init(), "lapis_hip_mult_%s" % _suffix(x))(int(x.shape[0]), _ptr(x), _ptr(y), _ptr(dst), _stream(stream)))
     return dst
 
 
 def div(x, y, dst, stream=None):
+    _holds("div", int(x.shape[0]), x, y, dst, like=x)
     check(getattr(init(), "lapis_hip_div_%s" % _suffix(x))(int(x.shape[0]), _ptr(x), _ptr(y), _ptr(dst), _stream(stream)))
     return dst
 
@@ -390,6 +435,7 @@ def fill(dst, value, stream=None):
 
 
 def copy(src, dst, stream=None):
+    _holds("copy", int(src.shape[0]), src, dst, like=src)
     check(getattr(init(), "lapis_hip_copy_%s" % _suffix(src))(int(src.shape[0]), _ptr(src), _ptr(dst), _stream(stream)))
     return dst
 
@@ -401,6 +447,12 @@ def scale(alpha, val, stream=None):
 
 def pcg(plan, n, pos, crd, val, b, dinv, tol, maxiter, x, work=None, stream=None):
     """CG of examples/pcg_solve.py on device buffers -> (iters, relres); x is filled in place."""
+    _indices("pcg", pos, crd)
+    _holds("pcg", n + 1, pos)
+    _holds("pcg", n, b, dinv, x, like=val)
+    _holds("pcg", 4 * n, work, like=val)
+    if not isinstance(crd, int) and not isinstance(val, int):
+        _holds("pcg", crd.numel(), val)
     lib = init()
     iters, relres = _u64(0), _dbl(0.0)
     check(lib.lapis_hip_pcg_f64_i32(plan.handle if plan is not None else None, n, _ptr(pos), _ptr(crd), _ptr(val),
@@ -411,6 +463,10 @@ def pcg(plan, n, pos, crd, val, b, dinv, tol, maxiter, x, work=None, stream=None
 
 def pcg_masked(plan, n, pos, crd, val, b, mask, d, tol, maxiter, x, work=None, stream=None):
     """Masked CG of examples/hitting_times.py:97 on device buffers -> (iters, relres)."""
+    _indices("pcg_masked", pos, crd)
+    _holds("pcg_masked", n + 1, pos)
+    _holds("pcg_masked", n, b, mask, d, x, like=val)
+    _holds("pcg_masked", 5 * n, work, like=val)
     lib = init()
     iters, relres = _u64(0), _dbl(0.0)
     check(lib.lapis_hip_pcg_masked_f64_i32(plan.handle if plan is not None else None, n, _ptr(pos), _ptr(crd),

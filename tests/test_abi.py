@@ -103,3 +103,29 @@ def test_nothing_under_the_package_reaches_for_the_oracle():
                 if re.search(r"liblapis_oracle|oracle\.oracle|from oracle|import oracle|lapis_oracle\.c", text):
                     offenders.append(os.path.join(root, name))
     assert offenders == []
+
+
+def test_the_python_binding_refuses_operands_the_kernels_would_overrun():
+    """lapis_amd.hip passes addresses and counts through ctypes: tensors that are too short, of another
+    element type, or not contiguous are refused before the library is asked for anything (no GPU needed)."""
+    import torch
+    from lapis_amd import hip
+    f64 = lambda n: torch.ones(n, dtype=torch.float64)
+    i32 = lambda n: torch.zeros(n, dtype=torch.int32)
+    x5, y4 = f64(5), f64(4)
+    for call in (lambda: hip.axpby(1.0, x5, 1.0, y4, x5), lambda: hip.dot_host(x5, y4), lambda: hip.mult(x5, y4, x5),
+                 lambda: hip.div(x5, x5, y4), lambda: hip.copy(x5, y4),
+                 lambda: hip.spmv(None, 5, 5, i32(6), i32(9), f64(9), y4, x5),        # x shorter than the columns
+                 lambda: hip.spmv(None, 5, 5, i32(5), i32(9), f64(9), x5, x5),        # positions for four rows
+                 lambda: hip.spmv(None, 5, 5, i32(6), i32(9), f64(8), x5, x5),        # fewer values than coordinates
+                 lambda: hip.pcg(None, 5, i32(6), i32(9), f64(9), x5, None, 0.0, 1, y4),
+                 lambda: hip.pcg(None, 5, i32(6), i32(9), f64(9), x5, None, 0.0, 1, x5, work=f64(19)),
+                 lambda: hip.copy(f64(10)[::2], x5),
+                 lambda: hip.spmm(5, 5, i32(6), i32(9), torch.ones(9), torch.ones(4, 3), torch.ones(5, 3))):
+        with pytest.raises(ValueError):
+            call()
+    for call in (lambda: hip.axpby(1.0, x5, 1.0, torch.ones(5), x5),
+                 lambda: hip.spmv(None, 5, 5, i32(6).long(), i32(9), f64(9), x5, x5),
+                 lambda: hip.spmv(None, 5, 5, i32(6), i32(9), f64(9), torch.ones(5), x5)):
+        with pytest.raises(TypeError):
+            call()
