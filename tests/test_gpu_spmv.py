@@ -533,7 +533,7 @@ def test_long_runs_of_empty_rows(gpu, oracle, kernel):
 
 
 def test_config1_at_its_full_size(gpu, oracle):
-    # BASELINE config 1 itself: the 5-point Laplacian on the 256 x 256 grid (65 536 rows, 326 656 non-zeros)
+    # the first benchmark configuration itself: the 5-point Laplacian on the 256 x 256 grid (65 536 rows, 326 656 non-zeros)
     A, x = gen.config1()
     assert (A.nrows, A.nnz) == (65536, 326656)
     want = np.zeros(A.nrows)
