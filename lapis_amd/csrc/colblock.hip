@@ -491,6 +491,11 @@ extern "C" int lapis_hip_csr_plan_build_colblock(lapis_hip_csr_plan *plan, const
   const lapis_hip_csr_stats &s = plan->stats;
   LAPIS_REQUIRE(s.nnz > 0, "csr_plan_build_colblock: the matrix has no non-zeros");
   LAPIS_REQUIRE(crd && val, "csr_plan_build_colblock: null coordinates or values");
+  // the kernels of both layouts step through the copy in trips of up to 16384 entries with int offsets,
+  // and the copy is padded: keep a margin below 2^31 so that no offset wraps
+  if (s.nnz > (int64_t)INT32_MAX - (1 << 20))
+    return set_error(LAPIS_HIP_ERR_NO_TILING, "csr_plan_build_colblock: %lld non-zeros leave no room below 2^31",
+                     (long long)s.nnz);
   if (layout == LAPIS_HIP_COLBLOCK_AUTO) layout = LAPIS_HIP_COLBLOCK_GROUP;
   int col_bits = 1;
   while ((1LL << col_bits) < s.ncols) ++col_bits;
