@@ -113,3 +113,47 @@ def test_config5_cg_fp64_full_size(gpu, oracle):
     true_relres = (torch.linalg.norm(r - Ax) / torch.linalg.norm(db)).item()
     assert abs(true_relres - relres) <= 1e-6 * relres
     assert np.isfinite(relres) and relres > 0
+
+
+@pytest.mark.parametrize("n, k, dtype", [(16_000_000, 133, torch.float32), (8_500_000, 192, torch.float64)])
+def test_spmv_close_to_the_int32_limit_of_the_positions(gpu, n, k, dtype):
+    """2.13 and 1.63 thousand million non-zeros (the positions are int32: 2^31 - 1 is the most a matrix can
+    hold): byte offsets beyond 2^32 and entry offsets next to 2^31 in every kernel family that takes the
+    matrix.  The matrix is made on the device (k entries per row at fixed offsets around the diagonal, wrapped)
+    and the expected product is taken by torch from the same arrays in double precision, slab by slab."""
+    rows = torch.arange(n, device="cuda", dtype=torch.int64)
+    offs = (torch.arange(k, device="cuda", dtype=torch.int64) - k // 2) * 37
+    pos = (torch.arange(n + 1, device="cuda", dtype=torch.int64) * k).to(torch.int32)
+    crd = torch.empty(n * k, device="cuda", dtype=torch.int32)
+    torch.manual_seed(5)
+    val = torch.rand(n * k, device="cuda", dtype=dtype) - 0.5
+    x = torch.rand(n, device="cuda", dtype=dtype) - 0.5
+    want = torch.empty(n, device="cuda", dtype=torch.float64)
+    scale = torch.empty(n, device="cuda", dtype=torch.float64)
+    slab = 1 << 20
+    for a in range(0, n, slab):
+        b = min(n, a + slab)
+        c, _ = torch.sort((rows[a:b, None] + offs[None, :]) % n, dim=1)
+        crd[a * k:b * k] = c.reshape(-1).to(torch.int32)
+        prod = val[a * k:b * k].view(b - a, k).double() * x[c].double()
+        want[a:b] = prod.sum(1)
+        scale[a:b] = prod.abs().sum(1)
+    del rows, c, prod
+    tol = TOL[np.dtype(np.float64 if dtype == torch.float64 else np.float32)]
+    for how in ("plan", "rowblock", "row split", "group"):
+        y = torch.zeros(n, device="cuda", dtype=dtype)
+        plan = gpu.CsrPlan(n, n, pos, crd, value_bytes=val.element_size())
+        try:
+            if how == "rowblock":
+                plan.set_kernel(2, 0)
+            elif how == "row split":
+                plan.set_kernel(3, 0)
+            elif how == "group":
+                plan.build_colblock(crd, val, layout="group")
+            gpu.spmv(plan, n, n, pos, crd, val, x, y)
+            plan.check()
+            err = ((y.double() - want).abs() / (scale + 1e-300)).max().item()
+            assert err <= tol, "%s (%s): error %g of the summed magnitudes" % (how, plan.kernel_name(), err)
+        finally:
+            plan.destroy()
+            del y
