@@ -157,3 +157,40 @@ def test_spmv_close_to_the_int32_limit_of_the_positions(gpu, n, k, dtype):
         finally:
             plan.destroy()
             del y
+
+
+def test_spmm_with_dense_operands_beyond_two_to_the_31_elements(gpu):
+    """B and C of 36 000 000 x 64 fp32 hold 2.3 thousand million elements each: element offsets into them do not fit
+    32 bits.  Four entries per row at fixed distances (wrapped); expected rows from torch in double precision on
+    every fifth slab of 2^20 rows and on the last one."""
+    torch.manual_seed(7)
+    n, per_row, k = 36_000_000, 4, 64
+    rows = torch.arange(n, device="cuda", dtype=torch.int64)
+    offs = torch.tensor([-1000003, -1, 1, 999983], device="cuda", dtype=torch.int64)
+    pos = (torch.arange(n + 1, device="cuda", dtype=torch.int64) * per_row).to(torch.int32)
+    c, _ = torch.sort((rows[:, None] + offs[None, :]) % n, dim=1)
+    crd = c.reshape(-1).to(torch.int32)
+    del c, rows
+    val = torch.rand(n * per_row, device="cuda", dtype=torch.float32) - 0.5
+    B = torch.rand(n, k, device="cuda", dtype=torch.float32) - 0.5
+    C = torch.zeros(n, k, device="cuda", dtype=torch.float32)
+    assert B.numel() > 2 ** 31
+    for with_plan in (False, True):
+        C.zero_()
+        plan = gpu.CsrPlan(n, n, pos, crd, value_bytes=4) if with_plan else None
+        gpu.spmm(n, n, pos, crd, val, B, C, plan=plan)
+        if plan is not None:
+            plan.destroy()
+        slab = 1 << 20
+        for a in list(range(0, n, slab))[::5] + [n - slab]:
+            b = min(n, a + slab)
+            cc = crd[a * per_row:b * per_row].view(b - a, per_row).long()
+            vv = val[a * per_row:b * per_row].view(b - a, per_row).double()
+            want = torch.zeros(b - a, k, device="cuda", dtype=torch.float64)
+            scale = torch.zeros_like(want)
+            for j in range(per_row):
+                t = vv[:, j, None] * B[cc[:, j]].double()
+                want += t
+                scale += t.abs()
+            err = ((C[a:b].double() - want).abs() / (scale + 1e-300)).max().item()
+            assert err <= TOL[np.dtype(np.float32)], "rows %d..%d: %g" % (a, b, err)
