@@ -135,3 +135,22 @@ def test_fused_axpby_dot_on_unaligned_buffers_stays_within_tolerance(gpu):
     want = 2.0 * x[1:] + -1.0 * y[1:]
     assert np.array_equal(dst.cpu().numpy(), want)
     assert abs(res.item() - float(want @ want)) <= 1e-12 * float(want @ want)
+
+
+def test_vector_kernels_beyond_two_to_the_31_elements(gpu):
+    """2.3 thousand million fp32 elements: the element count does not fit 32 bits.  Constant vectors, so that
+    every result is known exactly and the far end of the arrays is checked as well as the start."""
+    import torch
+    n = 2_300_000_000
+    x = torch.full((n,), 0.5, device="cuda", dtype=torch.float32)
+    y = torch.full((n,), 2.0, device="cuda", dtype=torch.float32)
+    d = torch.empty(n, device="cuda", dtype=torch.float32)
+    assert gpu.dot_host(x, y) == float(n)
+    gpu.axpby(2.0, x, 0.25, y, d)
+    assert d.min().item() == 1.5 and d.max().item() == 1.5 and d[n - 1].item() == 1.5
+    gpu.mult(x, y, d)
+    assert d.min().item() == 1.0 and d.max().item() == 1.0
+    gpu.fill(d, 3.0)
+    assert d.min().item() == 3.0 and d[n - 1].item() == 3.0
+    gpu.copy(x, d)
+    assert d.max().item() == 0.5 and d[n - 1].item() == 0.5
