@@ -39,8 +39,20 @@ class Refused(Exception):
 
 
 _NAME = r"%[\w.$-]+(?:#\d+)?"
+def _ieee(fn):
+    """Host scalars follow IEEE 754 as the emitted C++ does: x/0 is an infinity or a NaN, not an exception,
+    and the maximum of a NaN and a number is a NaN."""
+    def apply(a, b):
+        f32 = isinstance(a, numpy.float32) and isinstance(b, numpy.float32)
+        with numpy.errstate(all="ignore"):
+            r = fn(numpy.float32(a) if f32 else numpy.float64(a), numpy.float32(b) if f32 else numpy.float64(b))
+        return numpy.float32(r) if f32 else float(r)
+    return apply
+
+
 _FLOAT_BIN = {"arith.addf": lambda a, b: a + b, "arith.subf": lambda a, b: a - b, "arith.mulf": lambda a, b: a * b,
-              "arith.divf": lambda a, b: a / b, "arith.maximumf": max, "arith.minimumf": min}
+              "arith.divf": _ieee(numpy.divide), "arith.maximumf": _ieee(numpy.maximum),
+              "arith.minimumf": _ieee(numpy.minimum)}
 _INT_BIN = {"arith.addi": lambda a, b: a + b, "arith.subi": lambda a, b: a - b, "arith.muli": lambda a, b: a * b,
             "arith.divui": lambda a, b: a // b, "arith.divsi": lambda a, b: int(a / b) if b else 0,
             "arith.remui": lambda a, b: a % b, "arith.remsi": lambda a, b: a - b * int(a / b),
@@ -363,7 +375,15 @@ class Executor:
                 names = re.findall(_NAME, _split_colon(s.head)[0])
                 return op.split(".")[-1], [self._val(env, n) for n in names]
             can_overwrite = lambda nm: nm in owned and nm in defined_here and nm not in later[k]
-            results = self._statement(s, env, nests, owned, can_overwrite)
+            try:
+                results = self._statement(s, env, nests, owned, can_overwrite)
+            except ZeroDivisionError:
+                raise RuntimeError("%s: integer division by zero" % op)
+            except (AttributeError, TypeError, IndexError, KeyError) as e:
+                # an operand that is not what the operation's types say (a scalar where a tensor is named, ...):
+                # text MLIR's own verifier would not have let through
+                raise RuntimeError("%s: an operand does not have the type the operation declares (%s: %s)" % (
+                    op, type(e).__name__, e))
             names = []
             for r in s.results:
                 if ":" in r:
@@ -423,7 +443,8 @@ class Executor:
         if op == "arith.negf":
             return -vals[0]
         if op == "math.sqrt":
-            return numpy.sqrt(vals[0]) if isinstance(vals[0], numpy.floating) else float(numpy.sqrt(vals[0]))
+            with numpy.errstate(all="ignore"):  # the root of a negative number is a NaN
+                return numpy.sqrt(vals[0]) if isinstance(vals[0], numpy.floating) else float(numpy.sqrt(vals[0]))
         if op == "math.absf":
             return abs(vals[0])
         if op in ("arith.cmpi", "arith.cmpf"):

@@ -213,3 +213,28 @@ def test_operands_whose_sizes_do_not_agree_stop_on_the_host():
     with pytest.raises(ValueError, match="shorter buffer"):
         e.run("inner", [vec(np.ones(8)), vec(np.ones(5)), 0.0])
     assert "dot_host" not in fake_hip.calls and "dot" not in fake_hip.calls
+
+
+def test_host_scalars_follow_ieee_like_the_emitted_code():
+    """examples/pcg_solve.py with b = 0: r.r is 0, alpha = 0/0, relres = 0/0.  The emitted C++ computes NaNs and
+    leaves the loop after its first pass (NaN > tol is false); host scalars here must do the same, not raise."""
+    e = make(M.PCG)
+    A = spd(10, 4)
+    x, its, relres = e.run("pcg", [csr(A), vec(np.zeros(10)), vec(np.ones(10)), 1e-8, 50])
+    assert its == 1 and np.isnan(relres) and np.all(np.isnan(x.numpy()))
+    # an integer division by zero has no value to give: it is reported as such
+    e = make("""
+module {
+  func.func @f(%a: index, %b: index) -> index {
+    %q = arith.divui %a, %b : index
+    return %q : index
+  }
+}""")
+    assert e.run("f", [7, 2]) == [3]
+    with pytest.raises(RuntimeError, match="division by zero"):
+        e.run("f", [7, 0])
+    # an operand of the wrong kind (text that MLIR's verifier would refuse) is named, not leaked as a Python error
+    e = make(M.SPMV_THEN_AXPBY.replace("ins(%A, %x", "ins(%A, %a", 1))
+    with pytest.raises((RuntimeError, ex.Refused)):
+        e.check("residual")
+        e.run("residual", [csr(A), vec(np.ones(10)), vec(np.ones(10)), 1.0, 1.0])
