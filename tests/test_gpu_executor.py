@@ -27,7 +27,11 @@ def _csr_args(A):
 
 def _spd(n, seed):
     rng = np.random.Generator(np.random.PCG64(seed))
-    R = sp.random(n, n, density=min(1.0, 6.0 / n), random_state=np.random.RandomState(seed), format="csr")
+    # six random columns per row (scipy's sp.random draws from all n*n positions: a minute for n = 40 000)
+    per_row = min(n, 6)
+    cols = rng.integers(0, n, (n, per_row))
+    R = sp.csr_matrix((rng.random(n * per_row), cols.ravel(), np.arange(0, n * per_row + 1, per_row)), shape=(n, n))
+    R.sum_duplicates()
     S = R + R.T
     return sp.csr_matrix(S + sp.diags(np.asarray(abs(S).sum(axis=1)).ravel() + 1.0)), rng
 
