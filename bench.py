@@ -172,7 +172,7 @@ def cpu_baseline_spmv(A, x, budget_s=12.0):
     t0 = time.perf_counter()
     omp.spmv(A.pos, A.crd, A.val, x, y, parallel=True)
     one = time.perf_counter() - t0
-    reps = int(min(200, max(3, budget_s / max(one, 1e-6))))
+    reps = int(min(2000, max(3, budget_s / max(one, 1e-6))))
     t0 = time.perf_counter()
     for _ in range(reps):
         omp.spmv(A.pos, A.crd, A.val, x, y, parallel=True)
