@@ -364,24 +364,22 @@ __global__ __launch_bounds__(256) void long_row_list_kernel(int nrows, const int
 // key = (block << (col_bits + row_bits)) | (column << row_bits) | row in block: sorted,
 // the entries of a block come slice by slice and by column inside a slice.  A long row
 // (flag set) belongs to block nblocks_nat + rank / rows, as row rank % rows.
-// One wavefront per 1024 consecutive entries; the row of an entry comes from the positions by
-// bisection between the rows of the chunk's first and last entry (lanes 0 and 1 find those), so
-// the cost does not depend on how the entries are spread over the rows.
+// One wavefront per 1024 consecutive entries; the rows of the entries come from the positions
+// (rows_of_chunk), so the cost does not depend on how the entries are spread over the rows.
 __global__ __launch_bounds__(256) void colgroup_keys_kernel(int nrows, long long nnz, int row_bits, int col_bits,
                                                             int nblocks_nat, const int *__restrict__ long_flag,
                                                             const int *__restrict__ long_rank,
                                                             const int *__restrict__ pos,
                                                             const int *__restrict__ crd,
                                                             unsigned long long *__restrict__ keys) {
-  const int lane = threadIdx.x & 63;
-  const long long j0 = ((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * 1024;
+  __shared__ int s_rows[4][1024];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const long long j0 = ((long long)blockIdx.x * 4 + wave) * 1024;
   if (j0 >= nnz) return;
   const long long j1 = std::min(nnz, j0 + 1024);
-  int edge = 0;
-  if (lane < 2) edge = row_of_entry(pos, lane == 0 ? j0 : j1 - 1, 0, nrows - 1);
-  const int r_lo = __shfl(edge, 0, 64), r_hi = __shfl(edge, 1, 64);
+  rows_of_chunk(pos, nrows, j0, j1, s_rows[wave]);
   for (long long j = j0 + lane; j < j1; j += 64) {
-    const int row = row_of_entry(pos, j, r_lo, r_hi);
+    const int row = s_rows[wave][j - j0];
     long long v = row;  // position in the blocked numbering
     if (long_flag && long_flag[row]) v = ((long long)nblocks_nat << row_bits) + long_rank[row];
     const unsigned long long rb = (unsigned long long)(v >> row_bits);

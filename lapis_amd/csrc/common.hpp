@@ -151,4 +151,49 @@ __device__ __forceinline__ void wave_lds_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// rows[k] = row of non-zero j0 + k for the up to 1024 consecutive non-zeros [j0, j1) of one wavefront
+// (`rows` is that wavefront's own 1024 ints of LDS; all 64 lanes call).  Lanes 0 and 1 bisect the
+// positions for the rows of the first and last entry; every row in between that starts inside the
+// chunk leaves its number at its starting entry, and a running maximum over the chunk spreads the
+// numbers to the entries that follow (empty rows start at the entry of the next row that has one, which
+// wins the maximum).  A chunk that spans more than 2048 rows bisects entry by entry instead.  Works on
+// positions nobody has validated yet: every LDS index is checked, every row stays in [0, nrows).
+__device__ __forceinline__ void rows_of_chunk(const int *__restrict__ pos, int nrows, long long j0, long long j1,
+                                              int *rows) {
+  const int lane = threadIdx.x & 63;
+  const int n = (int)(j1 - j0);
+  int edge = 0;
+  if (lane < 2) edge = row_of_entry(pos, lane == 0 ? j0 : j1 - 1, 0, nrows - 1);
+  const int r_lo = __shfl(edge, 0, 64), r_hi = __shfl(edge, 1, 64);
+  if (r_hi - r_lo > 2048 || r_hi < r_lo) {
+    for (int k = lane; k < n; k += 64) rows[k] = row_of_entry(pos, j0 + k, r_lo, r_hi < r_lo ? r_lo : r_hi);
+    wave_lds_sync();
+    return;
+  }
+  for (int k = lane; k < 1024; k += 64) rows[k] = 0;
+  wave_lds_sync();
+  for (int r = r_lo + 1 + lane; r <= r_hi; r += 64) {
+    const long long at = (long long)pos[r] - j0;
+    if (at >= 0 && at < n) atomicMax(rows + at, r - r_lo);
+  }
+  wave_lds_sync();
+  int local[16];
+  int m = 0;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    m = max(m, rows[lane * 16 + i]);
+    local[i] = m;
+  }
+  int incl = m;
+  for (int o = 1; o < 64; o <<= 1) {
+    const int t = __shfl_up(incl, o, 64);
+    if (lane >= o) incl = max(incl, t);
+  }
+  int before = __shfl_up(incl, 1, 64);
+  if (lane == 0) before = 0;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) rows[lane * 16 + i] = r_lo + max(local[i], before);
+  wave_lds_sync();
+}
+
 }  // namespace lapis

@@ -357,14 +357,14 @@ __global__ __launch_bounds__(256) void row_stats_kernel(int nrows, const int *__
 //    much of x a wavefront's gathers wander over, small for stencils and bands, the whole
 //    vector for uniformly random columns;
 //  * how much of the matrix lies in a band around the diagonal (|column - row| <= 32 ... 256).
-// The row of an entry comes from the positions by bisection: lanes 0 and 1 find the rows of the
-// chunk's first and last entry, every lane then searches between those two.  The work is by
-// entries, so a row of a million entries costs what a million short rows cost.
+// The rows of a chunk's entries come from the positions (rows_of_chunk).  The work is by entries, so a
+// row of a million entries costs what a million short rows cost.
 __global__ __launch_bounds__(256) void entry_stats_kernel(int nrows, long long nnz, int ncols,
                                                           const int *__restrict__ pos,
                                                           const int *__restrict__ crd, DeviceStats *st) {
   __shared__ unsigned long long s_span[4], s_near[4][4];
   __shared__ int s_bad[4];
+  __shared__ int s_rows[4][1024];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const long long nchunks = (nnz + 1023) / 1024;
   unsigned cnt[4] = {0u, 0u, 0u, 0u};
@@ -373,16 +373,14 @@ __global__ __launch_bounds__(256) void entry_stats_kernel(int nrows, long long n
   for (long long chunk = (long long)blockIdx.x * 4 + wave; chunk < nchunks; chunk += (long long)gridDim.x * 4) {
     const long long j0 = chunk * 1024;
     const long long j1 = std::min(nnz, j0 + 1024);
-    int edge = 0;
-    if (lane < 2) edge = row_of_entry(pos, lane == 0 ? j0 : j1 - 1, 0, nrows - 1);
-    const int r_lo = __shfl(edge, 0, 64), r_hi = __shfl(edge, 1, 64);
+    rows_of_chunk(pos, nrows, j0, j1, s_rows[wave]);
     int mn = INT32_MAX, mx = INT32_MIN;
     for (long long j = j0 + lane; j < j1; j += 64) {
       const int cj = crd[j];
       if (cj < 0 || cj >= ncols) bad = 1;
       mn = std::min(mn, cj);
       mx = std::max(mx, cj);
-      const long long d = (long long)cj - row_of_entry(pos, j, r_lo, r_hi);
+      const long long d = (long long)cj - s_rows[wave][j - j0];
       const long long a = d < 0 ? -d : d;
       cnt[0] += a <= 32;
       cnt[1] += a <= 64;
@@ -394,6 +392,7 @@ __global__ __launch_bounds__(256) void entry_stats_kernel(int nrows, long long n
       mx = std::max(mx, __shfl_xor(mx, o, 64));
     }
     span += (unsigned long long)((long long)mx - (long long)mn);  // the same in every lane
+    wave_lds_sync();  // the next chunk's rows go into the same LDS
   }
   unsigned long long near[4];
 #pragma unroll
